@@ -28,7 +28,7 @@ class DevicePools:
         self.group_of_slot: Dict[int, int] = {}
         self.paged: Dict[int, object] = {}        # slot -> storage of a paged need
         self.state: Dict[int, object] = {}        # slot -> storage of a per-request need
-        for slot in sorted(needs):
+        for slot in sorted(needs, key=lambda key: key if isinstance(key, tuple) else (key,)):
             need = needs[slot]
             if not hasattr(need, "paged"):
                 raise TypeError(f"cache slot {slot}: {need!r} is no cache need (see parts/base.py)")

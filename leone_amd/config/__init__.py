@@ -1,2 +1,3 @@
 from .base import ConfigError, UnsupportedArchitecture, architecture_name, read_config_json
 from .qwen3 import Qwen3Config
+from .pamevik import PamevikConfig

@@ -57,6 +57,8 @@ class FieldReader:
 
     def positive_int(self, key: str, default: Any = _MISSING) -> int:
         value = self._get(key, default)
+        if value is None and default is None:
+            return None
         if isinstance(value, bool) or not isinstance(value, int):
             raise ConfigError(key, f"expected an integer, found {value!r}")
         if value <= 0:
@@ -104,7 +106,13 @@ def read_config_json(model_dir: str) -> dict:
 
 
 def architecture_name(raw: Mapping[str, Any]) -> str:
-    """The registry key of a config.json: ``architectures[0]``."""
+    """The registry key of a config.json: ``architectures[0]``, or ``architecture`` (one name) where a design's
+    files carry that key instead."""
+    single = raw.get("architecture")
+    if "architectures" not in raw and single is not None:
+        if not isinstance(single, str) or not single:
+            raise ConfigError("architecture", f"expected a name, found {single!r}")
+        return single
     names = raw.get("architectures")
     if not isinstance(names, list) or len(names) != 1 or not isinstance(names[0], str):
         raise ConfigError("architectures", f"expected a list with one name, found {names!r}")

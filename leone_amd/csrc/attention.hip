@@ -31,7 +31,8 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
                                       const T* __restrict__ k_pool, const T* __restrict__ v_pool,
                                       const int* __restrict__ positions, const int* __restrict__ row_entry,
                                       const int* __restrict__ block_table, int max_blocks, int q_heads,
-                                      int kv_heads, int head_dim, int page_tokens, float scale, int window) {
+                                      int kv_heads, int head_dim, int v_dim, int page_tokens, float scale, int window,
+                                      const float* __restrict__ gate, long gate_stride) {
     __shared__ float sm_m[kRowWaves];
     __shared__ float sm_l[kRowWaves];
     __shared__ float sm_acc[kRowWaves][kRowMaxHeadDim];
@@ -61,21 +62,16 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
             l = __builtin_nanf("");
             continue;
         }
-        const long head_base = (static_cast<long>(page) * kv_heads + kvh) * page_tokens * head_dim;
-        const T* kr = k_pool + head_base;
-        const T* vr = v_pool + head_base;
+        const T* kr = k_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * head_dim;
+        const T* vr = v_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * v_dim;
         const int token = j % page_tokens;
         float partial = 0.f;
         float vv[kRowDimsPerLane];
 #pragma unroll
         for (int i = 0; i < kRowDimsPerLane; ++i) {
             const int d = lane + i * kWave;
-            if (d < head_dim) {
-                partial = fmaf(qv[i], to_float(kr[key_offset(token, d, page_tokens)]), partial);
-                vv[i] = to_float(vr[value_offset(token, d, head_dim)]);
-            } else {
-                vv[i] = 0.f;
-            }
+            if (d < head_dim) partial = fmaf(qv[i], to_float(kr[key_offset(token, d, page_tokens)]), partial);
+            vv[i] = d < v_dim ? to_float(vr[value_offset(token, d, v_dim)]) : 0.f;
         }
         const float s = wave_sum(partial) * scale;
         const float m_new = fmaxf(m, s);
@@ -94,8 +90,10 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
     for (int i = 0; i < kRowDimsPerLane; ++i) sm_acc[wave][lane + i * kWave] = acc[i];
     __syncthreads();
 
-    T* orow = out + (static_cast<long>(row) * q_heads + head) * head_dim;
-    for (int d = threadIdx.x; d < head_dim; d += kRowThreads) {
+    T* orow = out + (static_cast<long>(row) * q_heads + head) * v_dim;
+    // an output gate of the head: the result times sigmoid(gate[row, head])
+    const float open = gate ? 1.0f / (1.0f + expf(-gate[static_cast<long>(row) * gate_stride + head])) : 1.0f;
+    for (int d = threadIdx.x; d < v_dim; d += kRowThreads) {
         float top = sm_m[0];
 #pragma unroll
         for (int w = 1; w < kRowWaves; ++w) top = fmaxf(top, sm_m[w]);
@@ -107,7 +105,7 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
             denom += sm_l[w] * wgt;
             num += sm_acc[w][d] * wgt;
         }
-        orow[d] = from_float<T>(num / denom);
+        orow[d] = from_float<T>(num / denom * open);
     }
 }
 
@@ -117,14 +115,17 @@ using namespace leone;
 
 extern "C" int leone_attention_rows(const void* q, void* out, const void* k_pool, const void* v_pool, int dtype,
                                     const int* positions, const int* row_entry, const int* block_table,
-                                    int max_blocks, int rows, int q_heads, int kv_heads, int head_dim,
-                                    int page_tokens, float scale, int window, hipStream_t stream) {
+                                    int max_blocks, int rows, int q_heads, int kv_heads, int head_dim, int v_dim,
+                                    int page_tokens, float scale, int window, const float* gate, long gate_stride,
+                                    hipStream_t stream) {
     LEONE_REQUIRE(dtype == kF32 || dtype == kBF16, "attention_rows: unknown element type %d", dtype);
     LEONE_REQUIRE(q && out && k_pool && v_pool && positions && row_entry && block_table, "attention_rows: null pointer");
     LEONE_REQUIRE(rows > 0 && q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
                   "attention_rows: rows %d, %d query heads over %d kv heads", rows, q_heads, kv_heads);
     LEONE_REQUIRE(q_heads <= 65535, "attention_rows: at most 65535 query heads");
     LEONE_REQUIRE(head_dim > 0 && head_dim <= kRowMaxHeadDim, "attention_rows: head_dim %d must be in 1..%d", head_dim, kRowMaxHeadDim);
+    LEONE_REQUIRE(v_dim > 0 && v_dim <= kRowMaxHeadDim, "attention_rows: value size %d must be in 1..%d", v_dim, kRowMaxHeadDim);
+    LEONE_REQUIRE(!gate || gate_stride >= q_heads, "attention_rows: gate rows of %ld for %d heads", gate_stride, q_heads);
     LEONE_REQUIRE(page_tokens > 0 && max_blocks > 0, "attention_rows: page_tokens %d and max_blocks %d must be positive", page_tokens, max_blocks);
     LEONE_REQUIRE(head_dim % 8 == 0 && page_tokens % 8 == 0,
                   "attention_rows: head_dim %d and page_tokens %d must be multiples of 8", head_dim, page_tokens);
@@ -134,12 +135,12 @@ extern "C" int leone_attention_rows(const void* q, void* out, const void* k_pool
         attention_rows_kernel<float><<<grid, kRowThreads, 0, stream>>>(
             static_cast<const float*>(q), static_cast<float*>(out), static_cast<const float*>(k_pool),
             static_cast<const float*>(v_pool), positions, row_entry, block_table, max_blocks, q_heads, kv_heads,
-            head_dim, page_tokens, scale, window);
+            head_dim, v_dim, page_tokens, scale, window, gate, gate_stride);
     else
         attention_rows_kernel<bf16_t><<<grid, kRowThreads, 0, stream>>>(
             static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_pool),
             static_cast<const bf16_t*>(v_pool), positions, row_entry, block_table, max_blocks, q_heads, kv_heads,
-            head_dim, page_tokens, scale, window);
+            head_dim, v_dim, page_tokens, scale, window, gate, gate_stride);
     LEONE_LAUNCH_CHECK("attention_rows");
     return 0;
 }

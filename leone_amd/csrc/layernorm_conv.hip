@@ -1,0 +1,329 @@
+// Row-wise kernels of layers that keep a short history of their own inputs:
+//
+//   add_layernorm     x += LayerNorm_a(delta) (if a delta comes), y = LayerNorm_b(x): the norm after one
+//                     sublayer, the residual sum and the norm before the next in one pass over the row
+//   entry_spans       first and last row of every entry of a step, from the row -> entry map
+//   causal_conv       out[t] = (in[t] if asked) + sum_j w[c, j] * in[t - (taps - 1) + j], per channel, the
+//                     rows before a portion taken from the request's state (its last taps - 1 inputs)
+//   causal_conv_state leaves the last taps - 1 inputs of every entry behind as the new state
+//   head_norm_gate    per head: (read-out / denominator) / rms * gain * act(gate)
+//   rms_mix           scale * sum_b rms(branch_b) * gain_b over the model width
+//   relu_squared      max(x, 0)^2
+//
+// Sums, means and variances are float whatever the storage type.
+#include "common.h"
+#include "leone_hip.h"
+
+#include <math.h>
+
+namespace leone {
+
+constexpr int kNormThreads = 256;
+constexpr int kMaxTaps = 16;
+
+// Mean and inverse deviation of n values read through f(i); every thread gets both.
+template <typename F>
+__device__ inline void mean_rstd(F value, int n, float eps, float* scratch, float& mean, float& rstd) {
+    float s = 0.f;
+    for (int i = threadIdx.x; i < n; i += kNormThreads) s += value(i);
+    mean = block_sum<kNormThreads>(s, scratch) / static_cast<float>(n);
+    float q = 0.f;
+    for (int i = threadIdx.x; i < n; i += kNormThreads) {
+        const float d = value(i) - mean;
+        q = fmaf(d, d, q);
+    }
+    const float var = block_sum<kNormThreads>(q, scratch) / static_cast<float>(n);
+    rstd = 1.0f / sqrtf(var + eps);
+}
+
+// One workgroup a row; the row lies in shared memory between the passes.
+template <typename TOut>
+__global__ void __launch_bounds__(kNormThreads)
+add_layernorm_kernel(float* __restrict__ x, const float* __restrict__ delta, AnyVec dw, AnyVec db, float deps,
+                     AnyVec w, AnyVec b, float eps, TOut* __restrict__ y, const int* __restrict__ rows, int hidden) {
+    extern __shared__ float row_buf[];
+    __shared__ float scratch[kNormThreads / kWave];
+    const long src = rows ? rows[blockIdx.x] : blockIdx.x;
+    float* xr = x + src * hidden;
+    if (delta) {
+        const float* dr = delta + src * hidden;
+        float mean = 0.f, rstd = 1.f;
+        if (dw.ptr) mean_rstd([&](int i) { return dr[i]; }, hidden, deps, scratch, mean, rstd);
+        for (int i = threadIdx.x; i < hidden; i += kNormThreads) {
+            float d = dr[i];
+            if (dw.ptr) d = (d - mean) * rstd * load_any(dw, i) + load_any(db, i);
+            const float t = xr[i] + d;
+            row_buf[i] = t;
+            if (!rows) xr[i] = t;
+        }
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += kNormThreads) row_buf[i] = xr[i];
+    }
+    if (!y) return;
+    __syncthreads();
+    float mean, rstd;
+    mean_rstd([&](int i) { return row_buf[i]; }, hidden, eps, scratch, mean, rstd);
+    TOut* yr = y + static_cast<long>(blockIdx.x) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += kNormThreads)
+        yr[i] = from_float<TOut>((row_buf[i] - mean) * rstd * load_any(w, i) + load_any(b, i));
+}
+
+__global__ void entry_spans_kernel(const int* __restrict__ row_entry, int rows, int* __restrict__ spans) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    const int e = row_entry[r];
+    if (r == 0 || row_entry[r - 1] != e) spans[2 * e] = r;
+    if (r == rows - 1 || row_entry[r + 1] != e) spans[2 * e + 1] = r + 1;
+}
+
+enum Activation : int { kActNone = 0, kActSigmoid = 1, kActSilu = 2 };
+
+__device__ inline float activate(float v, int act) {
+    if (act == kActNone) return v;
+    const float s = 1.0f / (1.0f + expf(-v));
+    return act == kActSigmoid ? s : v * s;
+}
+
+template <typename TIn, typename TOut>
+__global__ void causal_conv_kernel(const TIn* __restrict__ in, long in_stride, TOut* __restrict__ out, long out_stride,
+                                   AnyVec w, const float* __restrict__ state, const int* __restrict__ positions,
+                                   const int* __restrict__ row_entry, const int* __restrict__ entry_slots,
+                                   int channels, int taps, int add_input, int act) {
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    const int r = blockIdx.x;
+    if (c >= channels) return;
+    const int e = row_entry[r];
+    const int pos = positions[r];
+    int inside = 0;          // rows of this request that stand before row r in this step, as far as the taps reach
+    while (inside < taps - 1 && r - inside - 1 >= 0 && row_entry[r - inside - 1] == e) ++inside;
+    const float* mine = state + (static_cast<long>(entry_slots[e]) * (taps - 1)) * channels + c;
+    float acc = 0.f;
+    for (int back = taps - 1; back >= 0; --back) {          // oldest input first
+        float h;
+        if (pos - back < 0) h = 0.f;                          // before the sequence's start
+        else if (back <= inside) h = to_float(in[static_cast<long>(r - back) * in_stride + c]);
+        else h = mine[static_cast<long>(taps - 1 - (back - inside)) * channels];
+        acc = fmaf(load_any(w, static_cast<long>(c) * taps + (taps - 1 - back)), h, acc);
+    }
+    if (add_input) acc += to_float(in[static_cast<long>(r) * in_stride + c]);
+    out[static_cast<long>(r) * out_stride + c] = from_float<TOut>(activate(acc, act));
+}
+
+template <typename TIn>
+__global__ void causal_conv_state_kernel(const TIn* __restrict__ in, long in_stride, float* __restrict__ state,
+                                         const int* __restrict__ spans, const int* __restrict__ entry_slots,
+                                         const int* __restrict__ positions, int channels, int taps) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int e = blockIdx.y;
+    if (c >= channels) return;
+    const int first = spans[2 * e], n = spans[2 * e + 1] - first;
+    const int start = positions[first];
+    float* mine = state + (static_cast<long>(entry_slots[e]) * (taps - 1)) * channels + c;
+    float keep[kMaxTaps - 1];
+    for (int j = 0; j < taps - 1; ++j) {
+        const int back = taps - 1 - j;                        // how far before the end of the portion
+        if (back <= n) keep[j] = to_float(in[static_cast<long>(first + n - back) * in_stride + c]);
+        else if (start + n - back < 0) keep[j] = 0.f;
+        else keep[j] = mine[static_cast<long>(taps - 1 - (back - n)) * channels];
+    }
+    for (int j = 0; j < taps - 1; ++j) mine[static_cast<long>(j) * channels] = keep[j];
+}
+
+// One wave per (row, head).
+template <typename TOut>
+__global__ void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ dot, const float* __restrict__ top,
+                                      AnyVec gain, int gain_per_head, const float* __restrict__ gate, long gate_stride,
+                                      int act, float eps, TOut* __restrict__ out, int heads, int vdim) {
+    const int row = blockIdx.x;
+    const int head = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    if (head >= heads) return;
+    const long at = static_cast<long>(row) * heads + head;
+    const float* src = o + at * vdim;
+    float under = 1.f;
+    if (dot) under = fmaxf(fabsf(dot[at]), expf(-top[at])) + 1e-6f;
+    float ss = 0.f;
+    for (int j = lane; j < vdim; j += kWave) {
+        const float v = src[j] / under;
+        ss = fmaf(v, v, ss);
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(vdim) + eps);
+    TOut* dst = out + at * vdim;
+    for (int j = lane; j < vdim; j += kWave) {
+        float v = (src[j] / under) * inv;
+        if (gain.ptr) v *= load_any(gain, gain_per_head ? static_cast<long>(head) * vdim + j : j);
+        if (gate) v *= activate(gate[static_cast<long>(row) * gate_stride + static_cast<long>(head) * vdim + j], act);
+        dst[j] = from_float<TOut>(v);
+    }
+}
+
+constexpr int kMaxBranches = 4;
+struct Branches {
+    const float* rows[kMaxBranches];
+    AnyVec gain[kMaxBranches];
+};
+
+__global__ void __launch_bounds__(kNormThreads)
+rms_mix_kernel(Branches in, int branches, float eps, float scale, float* __restrict__ out, int hidden) {
+    __shared__ float scratch[kNormThreads / kWave];
+    const long row = blockIdx.x;
+    float inv[kMaxBranches];
+    for (int b = 0; b < branches; ++b) {
+        const float* src = in.rows[b] + row * hidden;
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < hidden; i += kNormThreads) ss = fmaf(src[i], src[i], ss);
+        inv[b] = 1.0f / sqrtf(block_sum<kNormThreads>(ss, scratch) / static_cast<float>(hidden) + eps);
+    }
+    for (int i = threadIdx.x; i < hidden; i += kNormThreads) {
+        float total = 0.f;
+        for (int b = 0; b < branches; ++b) total += in.rows[b][row * hidden + i] * inv[b] * load_any(in.gain[b], i);
+        out[row * hidden + i] = total * scale;
+    }
+}
+
+template <typename T>
+__global__ void relu_squared_kernel(const T* __restrict__ in, T* __restrict__ out, long n) {
+    for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * blockDim.x) {
+        const float v = fmaxf(to_float(in[i]), 0.f);
+        out[i] = from_float<T>(v * v);
+    }
+}
+
+// Per-head sigmoid gates on attention's output: out[r, h, :] *= sigmoid(gate[r * stride + h]).
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ out, const float* __restrict__ gate, long gate_stride, int heads, int vdim, long n) {
+    const long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x;
+    if (i >= n) return;
+    const long row = i / (static_cast<long>(heads) * vdim);
+    const int head = static_cast<int>((i / vdim) % heads);
+    out[i] = from_float<T>(to_float(out[i]) * activate(gate[row * gate_stride + head], kActSigmoid));
+}
+
+static bool known(int dtype) { return dtype == kF32 || dtype == kBF16; }
+
+}  // namespace leone
+
+using namespace leone;
+
+extern "C" int leone_add_layernorm(float* x, const float* delta, const void* dw, const void* db, float deps,
+                                   const void* w, const void* b, int w_dtype, float eps, void* y, int y_dtype,
+                                   const int* rows, int n_out, int hidden, hipStream_t stream) {
+    LEONE_REQUIRE(x && n_out > 0 && hidden > 0, "add_layernorm: needs a stream and positive sizes");
+    LEONE_REQUIRE(known(w_dtype) && known(y_dtype), "add_layernorm: unknown element type");
+    LEONE_REQUIRE((dw == nullptr) == (db == nullptr), "add_layernorm: the delta's gain and bias come together");
+    LEONE_REQUIRE(!dw || (delta && deps > 0.f), "add_layernorm: a norm of the delta needs a delta and an eps");
+    LEONE_REQUIRE(!y || (w && b && eps > 0.f), "add_layernorm: the output norm needs gain, bias and eps");
+    LEONE_REQUIRE(y || (delta && !rows), "add_layernorm: nothing to do");
+    LEONE_REQUIRE(static_cast<size_t>(hidden) * sizeof(float) <= 64 * 1024, "add_layernorm: rows of %d elements are too long", hidden);
+    const AnyVec vdw{dw, w_dtype}, vdb{db, w_dtype}, vw{w, w_dtype}, vb{b, w_dtype};
+    const size_t shared = static_cast<size_t>(hidden) * sizeof(float);
+    if (y_dtype == kF32)
+        add_layernorm_kernel<float><<<n_out, kNormThreads, shared, stream>>>(x, delta, vdw, vdb, deps, vw, vb, eps,
+                                                                            static_cast<float*>(y), rows, hidden);
+    else
+        add_layernorm_kernel<bf16_t><<<n_out, kNormThreads, shared, stream>>>(x, delta, vdw, vdb, deps, vw, vb, eps,
+                                                                             static_cast<bf16_t*>(y), rows, hidden);
+    LEONE_LAUNCH_CHECK("add_layernorm");
+    return 0;
+}
+
+extern "C" int leone_entry_spans(const int* row_entry, int rows, int* spans, hipStream_t stream) {
+    LEONE_REQUIRE(row_entry && spans && rows > 0, "entry_spans: needs a row map");
+    entry_spans_kernel<<<ceil_div(rows, 256), 256, 0, stream>>>(row_entry, rows, spans);
+    LEONE_LAUNCH_CHECK("entry_spans");
+    return 0;
+}
+
+extern "C" int leone_causal_conv(const void* in, int in_dtype, long in_stride, void* out, int out_dtype, long out_stride,
+                                 const void* w, int w_dtype, float* state, int write_state, const int* spans, int entries,
+                                 const int* positions, const int* row_entry, const int* entry_slots, int rows,
+                                 int channels, int taps, int add_input, int act, hipStream_t stream) {
+    LEONE_REQUIRE(in && out && w && state && positions && row_entry && entry_slots, "causal_conv: null pointer");
+    LEONE_REQUIRE(known(in_dtype) && known(out_dtype) && known(w_dtype), "causal_conv: unknown element type");
+    LEONE_REQUIRE(rows > 0 && channels > 0 && ceil_div(channels, 256) <= 65535 && in_stride >= channels && out_stride >= channels,
+                  "causal_conv: %d rows of %d channels", rows, channels);
+    LEONE_REQUIRE(taps >= 2 && taps <= kMaxTaps, "causal_conv: %d taps, the kernel takes 2..%d", taps, kMaxTaps);
+    LEONE_REQUIRE(act >= kActNone && act <= kActSilu, "causal_conv: unknown activation %d", act);
+    LEONE_REQUIRE(!write_state || (spans && entries > 0 && entries <= 65535), "causal_conv: the state's update needs the entries' spans");
+    const AnyVec vw{w, w_dtype};
+    const dim3 grid(rows, ceil_div(channels, 256));
+#define LEONE_CONV(TIN, TOUT)                                                                                         \
+    causal_conv_kernel<TIN, TOUT><<<grid, 256, 0, stream>>>(static_cast<const TIN*>(in), in_stride, static_cast<TOUT*>(out), \
+                                                            out_stride, vw, state, positions, row_entry, entry_slots, \
+                                                            channels, taps, add_input, act)
+    if (in_dtype == kF32 && out_dtype == kF32) LEONE_CONV(float, float);
+    else if (in_dtype == kF32) LEONE_CONV(float, bf16_t);
+    else if (out_dtype == kF32) LEONE_CONV(bf16_t, float);
+    else LEONE_CONV(bf16_t, bf16_t);
+#undef LEONE_CONV
+    LEONE_LAUNCH_CHECK("causal_conv");
+    if (write_state) {
+        const dim3 sgrid(ceil_div(channels, 256), entries);
+        if (in_dtype == kF32)
+            causal_conv_state_kernel<float><<<sgrid, 256, 0, stream>>>(static_cast<const float*>(in), in_stride, state, spans,
+                                                                       entry_slots, positions, channels, taps);
+        else
+            causal_conv_state_kernel<bf16_t><<<sgrid, 256, 0, stream>>>(static_cast<const bf16_t*>(in), in_stride, state, spans,
+                                                                        entry_slots, positions, channels, taps);
+        LEONE_LAUNCH_CHECK("causal_conv_state");
+    }
+    return 0;
+}
+
+extern "C" int leone_head_norm_gate(const float* o, const float* dot, const float* top, const void* gain, int gain_dtype,
+                                    int gain_per_head, const float* gate, long gate_stride, int act, float eps, void* out,
+                                    int out_dtype, int rows, int heads, int vdim, hipStream_t stream) {
+    LEONE_REQUIRE(o && out && rows > 0 && heads > 0 && vdim > 0, "head_norm_gate: needs read-outs and positive sizes");
+    LEONE_REQUIRE(known(out_dtype) && (!gain || known(gain_dtype)), "head_norm_gate: unknown element type");
+    LEONE_REQUIRE((dot == nullptr) == (top == nullptr), "head_norm_gate: the denominator's two parts come together");
+    LEONE_REQUIRE(act >= kActNone && act <= kActSilu && eps > 0.f, "head_norm_gate: activation %d, eps %g", act, eps);
+    LEONE_REQUIRE(rows <= 0x7fffffff && ceil_div(heads, 4) <= 65535, "head_norm_gate: too many heads");
+    const AnyVec vg{gain, gain_dtype};
+    const dim3 grid(rows, ceil_div(heads, 4));
+    if (out_dtype == kF32)
+        head_norm_gate_kernel<float><<<grid, 4 * kWave, 0, stream>>>(o, dot, top, vg, gain_per_head, gate, gate_stride, act, eps,
+                                                                     static_cast<float*>(out), heads, vdim);
+    else
+        head_norm_gate_kernel<bf16_t><<<grid, 4 * kWave, 0, stream>>>(o, dot, top, vg, gain_per_head, gate, gate_stride, act, eps,
+                                                                      static_cast<bf16_t*>(out), heads, vdim);
+    LEONE_LAUNCH_CHECK("head_norm_gate");
+    return 0;
+}
+
+extern "C" int leone_rms_mix(const float* const* branch_rows, const void* const* gains, int gain_dtype, int branches,
+                             float eps, float scale, float* out, int rows, int hidden, hipStream_t stream) {
+    LEONE_REQUIRE(branch_rows && gains && out && rows > 0 && hidden > 0, "rms_mix: needs branches and positive sizes");
+    LEONE_REQUIRE(branches >= 1 && branches <= kMaxBranches, "rms_mix: %d branches, the kernel takes 1..%d", branches, kMaxBranches);
+    LEONE_REQUIRE(known(gain_dtype) && eps > 0.f, "rms_mix: unknown gain type or eps");
+    Branches in{};
+    for (int b = 0; b < branches; ++b) {
+        LEONE_REQUIRE(branch_rows[b] && gains[b], "rms_mix: branch %d is missing", b);
+        in.rows[b] = branch_rows[b];
+        in.gain[b] = AnyVec{gains[b], gain_dtype};
+    }
+    rms_mix_kernel<<<rows, kNormThreads, 0, stream>>>(in, branches, eps, scale, out, hidden);
+    LEONE_LAUNCH_CHECK("rms_mix");
+    return 0;
+}
+
+extern "C" int leone_relu_squared(const void* in, void* out, int dtype, long n, hipStream_t stream) {
+    LEONE_REQUIRE(in && out && n > 0 && known(dtype), "relu_squared: needs values of a known type");
+    const long blocks = (n + 255) / 256;
+    const int grid = static_cast<int>(blocks < 8192 ? blocks : 8192);
+    if (dtype == kF32) relu_squared_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(in), static_cast<float*>(out), n);
+    else relu_squared_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(in), static_cast<bf16_t*>(out), n);
+    LEONE_LAUNCH_CHECK("relu_squared");
+    return 0;
+}
+
+extern "C" int leone_head_gate(void* out, int dtype, const float* gate, long gate_stride, int rows, int heads, int vdim,
+                               hipStream_t stream) {
+    LEONE_REQUIRE(out && gate && known(dtype) && rows > 0 && heads > 0 && vdim > 0, "head_gate: needs values and gates");
+    const long n = static_cast<long>(rows) * heads * vdim;
+    LEONE_REQUIRE((n + 255) / 256 <= 0x7fffffffL, "head_gate: too many values");
+    const int grid = static_cast<int>((n + 255) / 256);
+    if (dtype == kF32) head_gate_kernel<float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), gate, gate_stride, heads, vdim, n);
+    else head_gate_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), gate, gate_stride, heads, vdim, n);
+    LEONE_LAUNCH_CHECK("head_gate");
+    return 0;
+}

@@ -40,19 +40,23 @@ int leone_rope_table(float* cos_out, float* sin_out, double theta, int rotary_di
 // added up in order: a product cut along K.  The tables are [table_positions, rotary_dim / 2]; the first
 // rotary_dim elements of a head are rotated (rotary_dim even, at most head_dim), in pairs (i, i + rotary_dim / 2)
 // for pairing 0 (half split) or (2 i, 2 i + 1) for pairing 1 (adjacent); the rest is only normalised.
+// Value heads may have a size of their own (v_dim; 0: head_dim) and a row more columns than the heads
+// (row_width elements from row to row; 0: exactly the heads), which are left alone.
 int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_planes, long qkv_plane, void* q_out,
                              void* k_pool, void* v_pool, int dtype,
                              const void* q_gain, const void* k_gain, int gain_dtype, float eps,
                              const float* cos_table, const float* sin_table, int table_positions,
                              int rotary_dim, int pairing, const int* positions, const int* row_entry, const int* block_table, int max_blocks,
                              int rows, int q_heads, int kv_heads, int head_dim, int page_tokens, int write_cache,
-                             hipStream_t stream);
+                             int v_dim, long row_width, hipStream_t stream);
 
-// Attention of each query row over its request's cached keys [first, pos].
+// Attention of each query row over its request's cached keys [first, pos].  Values have v_dim elements a head
+// (the output's width); with `gate` (float, gate_stride elements from row to row, one a query head) a head's
+// result is multiplied by sigmoid(gate[row, head]).
 int leone_attention_rows(const void* q, void* out, const void* k_pool, const void* v_pool, int dtype,
                          const int* positions, const int* row_entry, const int* block_table, int max_blocks,
-                         int rows, int q_heads, int kv_heads, int head_dim, int page_tokens, float scale,
-                         int window, hipStream_t stream);
+                         int rows, int q_heads, int kv_heads, int head_dim, int v_dim, int page_tokens, float scale,
+                         int window, const float* gate, long gate_stride, hipStream_t stream);
 
 // The same on the matrix cores for bfloat16, the keys of a row cut into `splits` parts whose
 // partial results (part_acc: rows*q_heads*splits*head_dim floats, part_ml: rows*q_heads*splits*2)
@@ -195,4 +199,44 @@ int leone_sample_truncated_stages();
 int leone_sample_truncated_params();
 int leone_sample_truncated(const float* logits, const double* params, int* out, int rows, int vocab,
                            hipStream_t stream);
+
+// ---- layers that keep state of their own per request (layernorm_conv.hip, recurrent.hip) ----------------------
+// x += LayerNorm(delta; dw, db, deps) if delta comes (dw null: added as it is), then y = LayerNorm(x; w, b, eps)
+// if y is wanted.  With `rows` (indices) row i of y comes from row rows[i] and x is not written.
+int leone_add_layernorm(float* x, const float* delta, const void* dw, const void* db, float deps, const void* w,
+                        const void* b, int w_dtype, float eps, void* y, int y_dtype, const int* rows, int n_out,
+                        int hidden, hipStream_t stream);
+// spans[2e], spans[2e + 1]: first row and end of entry e (an entry's rows are consecutive).
+int leone_entry_spans(const int* row_entry, int rows, int* spans, hipStream_t stream);
+// A causal convolution over time per channel, w [channels, taps] with the last tap on the current row; the
+// rows before a portion come from state [slots, taps - 1, channels] (float), which is brought up to date if asked.
+// act: 0 none, 1 sigmoid, 2 silu.
+int leone_causal_conv(const void* in, int in_dtype, long in_stride, void* out, int out_dtype, long out_stride,
+                      const void* w, int w_dtype, float* state, int write_state, const int* spans, int entries,
+                      const int* positions, const int* row_entry, const int* entry_slots, int rows, int channels,
+                      int taps, int add_input, int act, hipStream_t stream);
+// out = (o / (max(|dot|, exp(-top)) + 1e-6) if dot comes) / rms over vdim * gain * act(gate), head by head.
+int leone_head_norm_gate(const float* o, const float* dot, const float* top, const void* gain, int gain_dtype,
+                         int gain_per_head, const float* gate, long gate_stride, int act, float eps, void* out,
+                         int out_dtype, int rows, int heads, int vdim, hipStream_t stream);
+// out = scale * sum over branches of rms(branch) * gain.
+int leone_rms_mix(const float* const* branch_rows, const void* const* gains, int gain_dtype, int branches, float eps,
+                  float scale, float* out, int rows, int hidden, hipStream_t stream);
+int leone_relu_squared(const void* in, void* out, int dtype, long n, hipStream_t stream);
+int leone_head_gate(void* out, int dtype, const float* gate, long gate_stride, int rows, int heads, int vdim,
+                    hipStream_t stream);
+// The matrix-memory recurrences (see recurrent.hip); key sizes up to leone_scan_max_dim().
+int leone_scan_max_dim();
+int leone_outer_scan(const float* proj, long stride, int q_off, int k_off, int v_off, int i_off, int f_off,
+                     const void* i_bias, const void* f_bias, int bias_dtype, float cap, const float* decay,
+                     float q_scale, float k_scale, const float* cos_table, const float* sin_table, int rotary_dim,
+                     int table_positions, float* state, long slot_stride, int write_state, const int* spans,
+                     const int* entry_slots, const int* positions, int entries, float* out, float* dot, float* top,
+                     int heads, int dim, int vdim, hipStream_t stream);
+int leone_delta_scan(const float* qkv, long stride, int q_off, int k_off, int v_off, const float* beta,
+                     long beta_stride, const float* step, long step_stride, const void* rate_log,
+                     const void* step_bias, int vec_dtype, float q_scale, float unit_eps, float* state,
+                     long slot_stride, int write_state, const int* spans, const int* entry_slots,
+                     const int* positions, int entries, float* out, int heads, int kv_heads, int dim, int vdim,
+                     hipStream_t stream);
 }

@@ -242,19 +242,23 @@ __global__ void qk_norm_rope_write_kernel(
     AnyVec q_gain, AnyVec k_gain, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int table_positions, const int* __restrict__ positions,
     const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
-    int q_heads, int kv_heads, int head_dim, int page_tokens, int write_cache, int rotary_half, int pairing) {
+    int q_heads, int kv_heads, int head_dim, int page_tokens, int write_cache, int rotary_half, int pairing,
+    int v_dim, long row_width) {
     const int row = blockIdx.x;
     const int head = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
     const int lane = threadIdx.x % kWave;
     const int heads_total = q_heads + (write_cache ? 2 * kv_heads : 0);
     if (head >= heads_total) return;
-    const int half = head_dim / 2;
-    const int qkv_width = (q_heads + 2 * kv_heads) * head_dim;
-    const TIn* src = qkv + static_cast<long>(row) * qkv_width + static_cast<long>(head) * head_dim;
-    const int pos = positions[row];
-
     const bool is_q = head < q_heads;
     const bool is_k = !is_q && head < q_heads + kv_heads;
+    // a value head may have a size of its own (v_dim); a row may hold more columns than the heads (row_width)
+    const int size = (is_q || is_k) ? head_dim : v_dim;
+    const int half = size / 2;
+    const long head_at = (is_q || is_k) ? static_cast<long>(head) * head_dim
+                                        : static_cast<long>(q_heads + kv_heads) * head_dim + static_cast<long>(head - q_heads - kv_heads) * v_dim;
+    const TIn* src = qkv + static_cast<long>(row) * row_width + head_at;
+    const int pos = positions[row];
+
     // Where element d of this head goes: q rows are plain; keys and values use the cache's packed layout.
     T* dst;
     int kind = 0;  // 0 plain, 1 key page, 2 value page
@@ -265,12 +269,12 @@ __global__ void qk_norm_rope_write_kernel(
         const int kvh = is_k ? head - q_heads : head - q_heads - kv_heads;
         const int page = block_table[static_cast<long>(row_entry[row]) * max_blocks + pos / page_tokens];
         if (page < 0) return;  // host reserves pages before the launch
-        dst = (is_k ? k_pool : v_pool) + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * head_dim;
+        dst = (is_k ? k_pool : v_pool) + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * size;
         kind = is_k ? 1 : 2;
         token = pos % page_tokens;
     }
     auto place = [&](int d) -> long {
-        return kind == 0 ? d : kind == 1 ? key_offset(token, d, page_tokens) : value_offset(token, d, head_dim);
+        return kind == 0 ? d : kind == 1 ? key_offset(token, d, page_tokens) : value_offset(token, d, size);
     };
 
     // the two elements of pair p
@@ -704,7 +708,14 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_
                                         int rotary_dim, int pairing,
                                         const int* positions, const int* row_entry, const int* block_table,
                                         int max_blocks, int rows, int q_heads, int kv_heads, int head_dim,
-                                        int page_tokens, int write_cache, hipStream_t stream) {
+                                        int page_tokens, int write_cache, int v_dim, long row_width, hipStream_t stream) {
+    if (v_dim <= 0) v_dim = head_dim;
+    const long heads_width = static_cast<long>(q_heads + kv_heads) * head_dim + static_cast<long>(kv_heads) * v_dim;
+    if (row_width <= 0) row_width = heads_width;
+    LEONE_REQUIRE(row_width >= heads_width, "qk_norm_rope_write: rows of %ld elements do not hold the heads (%ld)", row_width, heads_width);
+    LEONE_REQUIRE(v_dim % 2 == 0 && v_dim <= 2 * kWave * kMaxPairsPerLane, "qk_norm_rope_write: value size %d must be even and at most %d",
+                  v_dim, 2 * kWave * kMaxPairsPerLane);
+    LEONE_REQUIRE(qkv_planes == 1 || row_width == heads_width, "qk_norm_rope_write: planes come without further columns");
     if (check_dtype(dtype, "qk_norm_rope_write") || check_dtype(gain_dtype, "qk_norm_rope_write gain") ||
         check_dtype(qkv_dtype, "qk_norm_rope_write input"))
         return 1;
@@ -734,7 +745,7 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_
                          (!write_cache || (reinterpret_cast<uintptr_t>(k_pool) % run_bytes == 0 && page_tokens % 8 == 0));
     const bool tables_aligned = (!q_gain || (reinterpret_cast<uintptr_t>(q_gain) % 32 == 0 && reinterpret_cast<uintptr_t>(k_gain) % 32 == 0)) &&
                                 (!cos_table || (reinterpret_cast<uintptr_t>(cos_table) % 32 == 0 && reinterpret_cast<uintptr_t>(sin_table) % 32 == 0));
-    if (whole_head && head_dim % 16 == 0 && head_dim <= 128 && aligned && tables_aligned && static_cast<long>(rows) * (q_heads + 2 * kv_heads) * 8 < 0x7fffffffL * 256) {
+    if (whole_head && v_dim == head_dim && row_width == heads_width && head_dim % 16 == 0 && head_dim <= 128 && aligned && tables_aligned && static_cast<long>(rows) * (q_heads + 2 * kv_heads) * 8 < 0x7fffffffL * 256) {
 #define LEONE_RUNS_ARGS                                                                                             \
     qkv, qkv_planes, qkv_plane, q_out, k_pool, v_pool, qg, kg, eps, cos_table, sin_table, table_positions, positions, \
         row_entry, block_table, max_blocks, rows, q_heads, kv_heads, page_tokens, write_cache, stream
@@ -760,7 +771,8 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_
     qk_norm_rope_write_kernel<TIN, T><<<grid, waves_per_block * kWave, 0, stream>>>(                                \
         static_cast<const TIN*>(qkv), qkv_planes, qkv_plane, static_cast<T*>(q_out), static_cast<T*>(k_pool),       \
         static_cast<T*>(v_pool), qg, kg, eps, cos_table, sin_table, table_positions, positions, row_entry,          \
-        block_table, max_blocks, q_heads, kv_heads, head_dim, page_tokens, write_cache, cos_table ? rotary_dim / 2 : 0, pairing)
+        block_table, max_blocks, q_heads, kv_heads, head_dim, page_tokens, write_cache, cos_table ? rotary_dim / 2 : 0, pairing, \
+        v_dim, row_width)
     if (dtype == kF32) LEONE_QK_ANY(float, float);
     else if (qkv_dtype == kF32) LEONE_QK_ANY(float, bf16_t);
     else LEONE_QK_ANY(bf16_t, bf16_t);

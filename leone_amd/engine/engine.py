@@ -431,6 +431,9 @@ class Engine:
             # one pool of memory for all recordings: they run one after the other on one stream, and what a
             # replay leaves in its logits is copied out before the next replay begins
             # (errors of the capture are this thread's: an engine in another thread goes on with its own work)
+            # a context of its own: what the parts derived on the device for the run above (``StepContext.spans``)
+            # is derived again inside the recording, in the recording's memory
+            context = state.context(bucket)
             with torch.cuda.graph(graph, pool=self._graph_pool, capture_error_mode="thread_local"), ops.one_stream():
                 recorded_logits = self.model.forward(state.tokens, context, caches)
             state.recordings[bucket] = (graph, recorded_logits)

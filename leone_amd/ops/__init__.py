@@ -80,16 +80,24 @@ class one_stream:
         return False
 
 
-def cache_dims(k_pool: torch.Tensor, v_pool: torch.Tensor):
-    """(pages, kv_heads, page_tokens, head_dim) of a key/value pool pair in the packed cache layout:
-    keys ``[pages, kv_heads, head_dim/8, page_tokens, 8]``, values ``[pages, kv_heads, page_tokens/8, head_dim, 8]``."""
+def cache_dims_kv(k_pool: torch.Tensor, v_pool: torch.Tensor):
+    """(pages, kv_heads, page_tokens, head_dim, value_dim) of a key/value pool pair in the packed cache layout:
+    keys ``[pages, kv_heads, head_dim/8, page_tokens, 8]``, values ``[pages, kv_heads, page_tokens/8, value_dim, 8]``."""
     if k_pool.dim() != 5 or k_pool.shape[4] != 8:
         raise KernelError(f"key pool must be [pages, kv_heads, head_dim/8, page_tokens, 8], found {tuple(k_pool.shape)}")
     pages, kv_heads, d8, page_tokens, _ = k_pool.shape
-    if page_tokens % 8 or tuple(v_pool.shape) != (pages, kv_heads, page_tokens // 8, d8 * 8, 8):
-        raise KernelError(f"value pool must be [pages, kv_heads, page_tokens/8, head_dim, 8] matching the key pool "
+    if page_tokens % 8 or v_pool.dim() != 5 or (tuple(v_pool.shape[:3]) + (v_pool.shape[4],)) != (pages, kv_heads, page_tokens // 8, 8):
+        raise KernelError(f"value pool must be [pages, kv_heads, page_tokens/8, value_dim, 8] matching the key pool "
                           f"{tuple(k_pool.shape)}, found {tuple(v_pool.shape)}")
-    return pages, kv_heads, page_tokens, d8 * 8
+    return pages, kv_heads, page_tokens, d8 * 8, v_pool.shape[3]
+
+
+def cache_dims(k_pool: torch.Tensor, v_pool: torch.Tensor):
+    """(pages, kv_heads, page_tokens, head_dim) of a pool pair whose values have the keys' size."""
+    pages, kv_heads, page_tokens, head_dim, value_dim = cache_dims_kv(k_pool, v_pool)
+    if value_dim != head_dim:
+        raise KernelError(f"values of {value_dim} elements beside keys of {head_dim}: this kernel takes one size for both")
+    return pages, kv_heads, page_tokens, head_dim
 
 
 def pack_keys(k: torch.Tensor) -> torch.Tensor:
@@ -201,29 +209,33 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim:
                        row_entry: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                        k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor], write_cache: bool = True,
                        out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
-                       pairing: str = "half_split") -> torch.Tensor:
+                       pairing: str = "half_split", value_dim: Optional[int] = None) -> torch.Tensor:
     """Splits the fused projection, normalises and rotates q and k heads, writes k and v into the cache.
     ``qkv`` is ``[rows, width]`` of the cache's type, or float32 (also as planes ``[p, rows, width]`` whose
     sum, in order, is meant: a product cut along K) with ``out_dtype`` naming the type of q and the cache.
     The rotation's shape comes with its tables (``_rotation_shape``): their width says how much of a head is
-    rotated, ``pairing`` which elements go together."""
+    rotated, ``pairing`` which elements go together.  ``value_dim``: the value heads' own size (then a row may
+    also hold further columns behind the heads, which are left alone)."""
     planes = qkv.shape[0] if qkv.dim() == 3 else 1
     rows, width = qkv.shape[-2:]
     kind = out_dtype or qkv.dtype
     if qkv.dtype != kind and qkv.dtype != torch.float32:
         raise KernelError(f"qk_norm_rope_write: input {qkv.dtype} for outputs of {kind}")
-    if width != (q_heads + 2 * kv_heads) * head_dim:
-        raise KernelError(f"qk_norm_rope_write: width {width} is not ({q_heads}+2*{kv_heads})*{head_dim}")
+    general = value_dim is not None
+    value_dim = head_dim if value_dim is None else int(value_dim)
+    heads_width = (q_heads + kv_heads) * head_dim + kv_heads * value_dim
+    if width != heads_width and not (general and width > heads_width and planes == 1):
+        raise KernelError(f"qk_norm_rope_write: width {width} is not ({q_heads}+{kv_heads})*{head_dim}+{kv_heads}*{value_dim}")
     if out is None:
         out = torch.empty((rows, q_heads * head_dim), dtype=kind, device=qkv.device)
     max_blocks = page_tokens = 0
     if write_cache:
         if k_pool is None or v_pool is None or block_table is None or row_entry is None:
             raise KernelError("qk_norm_rope_write: a cache write needs pools, a block table and a row map")
-        pages, pool_heads, page_tokens, pool_dim = cache_dims(k_pool, v_pool)
-        if (pool_heads, pool_dim) != (kv_heads, head_dim):
-            raise KernelError(f"qk_norm_rope_write: pool shape {tuple(k_pool.shape)} does not fit "
-                              f"{kv_heads} heads of {head_dim}")
+        pages, pool_heads, page_tokens, pool_dim, pool_vdim = cache_dims_kv(k_pool, v_pool)
+        if (pool_heads, pool_dim, pool_vdim) != (kv_heads, head_dim, value_dim):
+            raise KernelError(f"qk_norm_rope_write: pool shapes {tuple(k_pool.shape)}, {tuple(v_pool.shape)} do not fit "
+                              f"{kv_heads} heads of {head_dim} and {value_dim}")
         max_blocks = block_table.shape[1]
     table_positions, rotary_dim, pairing_code = _rotation_shape("qk_norm_rope_write", head_dim, cos, sin, pairing)
     gain_code = _code(q_gain, "q gain") if q_gain is not None else F32
@@ -238,25 +250,39 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim:
          rotary_dim, pairing_code, _dev(positions, "positions", torch.int32, (rows,)),
          _dev(row_entry if write_cache else None, "row map", torch.int32, (rows,)),
          _dev(block_table if write_cache else None, "block table", torch.int32), max_blocks, rows, q_heads,
-         kv_heads, head_dim, page_tokens, 1 if write_cache else 0, _stream())
+         kv_heads, head_dim, page_tokens, 1 if write_cache else 0, value_dim, width, _stream())
     return out
+
+
+def _strided_rows(t: Optional[torch.Tensor], what: str, rows: int, columns: int, dtype=torch.float32):
+    """(address, elements from row to row) of a 2-D float view whose rows may be slices of wider rows."""
+    if t is None:
+        return 0, 0
+    if not t.is_cuda or t.dtype != dtype or t.dim() != 2 or t.shape[0] != rows or t.shape[1] < columns \
+            or (t.shape[1] > 1 and t.stride(1) != 1) or t.stride(0) < t.shape[1]:
+        raise KernelError(f"{what}: expected {dtype} [{rows}, >= {columns}] with unit stride along a row, found "
+                          f"{t.dtype} {tuple(t.shape)} strides {t.stride()} on {t.device}")
+    return t.data_ptr(), t.stride(0)
 
 
 def attention_rows(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
                    row_entry: torch.Tensor, block_table: torch.Tensor, q_heads: int, scale: float,
-                   window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Each query row attends its request's cached keys up to its own position."""
+                   window: int = 0, out: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Each query row attends its request's cached keys up to its own position.  The result has the values'
+    size a head.  ``gate``: float32 ``[rows, >= q_heads]`` (a view into a wider row is fine, unit stride along the
+    heads): head h of row r is multiplied by sigmoid(gate[r, h])."""
     rows = q.shape[0]
-    pages, kv_heads, page_tokens, head_dim = cache_dims(k_pool, v_pool)
+    pages, kv_heads, page_tokens, head_dim, value_dim = cache_dims_kv(k_pool, v_pool)
     if q.shape[1] != q_heads * head_dim:
         raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
     if out is None:
-        out = torch.empty_like(q)
-    call("leone_attention_rows", _dev(q, "attention q"), _dev(out, "attention out", q.dtype, q.shape),
+        out = torch.empty((rows, q_heads * value_dim), dtype=q.dtype, device=q.device)
+    gate_at, gate_stride = _strided_rows(gate, "attention gate", rows, q_heads)
+    call("leone_attention_rows", _dev(q, "attention q"), _dev(out, "attention out", q.dtype, (rows, q_heads * value_dim)),
          _dev(k_pool, "k pool", q.dtype), _dev(v_pool, "v pool", q.dtype), _code(q, "attention q"),
          _dev(positions, "positions", torch.int32, (rows,)), _dev(row_entry, "row map", torch.int32, (rows,)),
          _dev(block_table, "block table", torch.int32), block_table.shape[1], rows, q_heads, kv_heads, head_dim,
-         page_tokens, float(scale), int(window), _stream())
+         value_dim, page_tokens, float(scale), int(window), gate_at, gate_stride, _stream())
     return out
 
 
@@ -1044,3 +1070,206 @@ def sample_truncated(logits: torch.Tensor, draws) -> torch.Tensor:
 
 
 __all__ = [name for name in dir() if not name.startswith("_")]
+
+
+# ---- layers that keep state of their own per request ---------------------------------------------------------
+ACTIVATIONS = {None: 0, "none": 0, "sigmoid": 1, "silu": 2}
+
+
+class NormedDelta:
+    """What a sublayer adds to the stream, still to be normalised: ``norm`` (a norm part) is applied to
+    ``rows`` (float32 ``[rows, hidden]``) before the sum.  The norm part that runs next takes it in place of a
+    delta and does both in one pass (``add_layernorm``); any other consumer asks for ``materialize()``."""
+
+    def __init__(self, rows: torch.Tensor, norm):
+        self.rows, self.norm = rows, norm
+
+    def materialize(self) -> torch.Tensor:
+        return self.norm.apply(self.rows)
+
+
+def add_layernorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional[torch.Tensor],
+                  bias: Optional[torch.Tensor], eps: float, out_dtype: Optional[torch.dtype],
+                  rows: Optional[torch.Tensor] = None, delta_norm: Optional[tuple] = None) -> Optional[torch.Tensor]:
+    """x += delta, where ``delta_norm`` = (gain, bias, eps) says that the delta goes through a layer norm of its
+    own first; then y = (x - mean) / sqrt(var + eps) * gain + bias in ``out_dtype`` (None: no y, only the sum).
+    With ``rows`` y[i] comes from row rows[i] and x is not written.  Means and variances are float."""
+    n, hidden = x.shape
+    n_out = n if rows is None else rows.numel()
+    if delta is not None and delta.dtype != torch.float32:
+        delta = delta.float()
+    y = torch.empty((n_out, hidden), dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    vectors = [v for v in (gain, bias) + tuple(delta_norm[:2] if delta_norm else ()) if v is not None]
+    if len({v.dtype for v in vectors}) > 1:
+        raise KernelError("add_layernorm: gains and biases must share one type")
+    call("leone_add_layernorm", _dev(x, "stream", torch.float32), _dev(delta, "delta", torch.float32, (n, hidden)),
+         _dev(delta_norm[0], "delta gain", None, (hidden,)) if delta_norm else 0,
+         _dev(delta_norm[1], "delta bias", None, (hidden,)) if delta_norm else 0,
+         float(delta_norm[2]) if delta_norm else 0.0,
+         _dev(gain, "gain", None, (hidden,)), _dev(bias, "bias", None, (hidden,)),
+         _code(vectors[0], "gain") if vectors else F32, float(eps), _dev(y, "normed rows"),
+         _CODES[out_dtype] if out_dtype is not None else F32,
+         _dev(rows, "rows", torch.int32) if rows is not None else 0, n_out, hidden, _stream())
+    return y
+
+
+def entry_spans(step) -> torch.Tensor:
+    """int32 ``[entries, 2]`` on the device: first row and end of every entry's rows in the step, made once a
+    step from the row -> entry map (so that it is there too when a step is replayed from a recording)."""
+    spans = getattr(step, "spans", None)
+    if spans is None:
+        entries = step.entry_slots.numel()
+        spans = torch.empty((entries, 2), dtype=torch.int32, device=step.row_entry.device)
+        call("leone_entry_spans", _dev(step.row_entry, "row map", torch.int32, (step.rows,)), step.rows,
+             _dev(spans, "spans"), _stream())
+        step.spans = spans
+    return spans
+
+
+def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, step, out_dtype: torch.dtype,
+                add_input: bool = False, activation: Optional[str] = None, write_state: bool = True) -> torch.Tensor:
+    """out[t, c] = (x[t, c] if ``add_input``) + sum_j weight[c, j] * x[t - (taps - 1) + j, c], then the
+    activation; rows before a portion come from ``state`` (float32 ``[slots, taps - 1, channels]``: a request's
+    last inputs), zeros before position 0.  ``x`` may be a column slice of wider rows.  Leaves the state
+    brought up to date unless told not to."""
+    rows, channels = x.shape
+    taps = weight.shape[1]
+    if tuple(weight.shape) != (channels, taps) or x.dim() != 2 or x.stride(1) != 1:
+        raise KernelError(f"causal_conv: weight {tuple(weight.shape)} for rows of {channels} channels")
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (taps - 1, channels):
+        raise KernelError(f"causal_conv: state {tuple(state.shape)} is not [slots, {taps - 1}, {channels}] float32")
+    if not x.is_cuda:
+        raise KernelError("causal_conv: tensor is not on the GPU")
+    out = torch.empty((rows, channels), dtype=out_dtype, device=x.device)
+    spans = entry_spans(step)
+    call("leone_causal_conv", x.data_ptr(), _code(x, "conv input"), x.stride(0), _dev(out, "conv out"), _CODES[out_dtype],
+         channels, _dev(weight, "conv weight"), _code(weight, "conv weight"), _dev(state, "conv state"),
+         1 if write_state else 0, _dev(spans, "spans"), spans.shape[0],
+         _dev(step.positions, "positions", torch.int32, (rows,)), _dev(step.row_entry, "row map", torch.int32, (rows,)),
+         _dev(step.entry_slots, "slots", torch.int32), rows, channels, taps, 1 if add_input else 0,
+         ACTIVATIONS[activation], _stream())
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, heads: int, vdim: int, eps: float, out_dtype: torch.dtype,
+                   gain: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                   activation: Optional[str] = None, denominator: Optional[tuple] = None) -> torch.Tensor:
+    """Head by head: o (float32 ``[rows, heads * vdim]``), divided by max(|dot|, exp(-top)) + 1e-6 if
+    ``denominator`` = (dot, top) (float32 ``[rows, heads]``) comes, over its root mean square, times ``gain``
+    (``[heads * vdim]``, or ``[vdim]`` shared by the heads), times activation(gate) (float32 rows of heads * vdim,
+    possibly a slice of wider rows)."""
+    rows = o.shape[0]
+    out = torch.empty((rows, heads * vdim), dtype=out_dtype, device=o.device)
+    per_head = 0
+    if gain is not None:
+        if gain.numel() == heads * vdim and heads > 1:
+            per_head = 1
+        elif gain.numel() != vdim:
+            raise KernelError(f"head_norm_gate: a gain of {gain.numel()} for {heads} heads of {vdim}")
+    gate_at, gate_stride = _strided_rows(gate, "head_norm_gate gate", rows, heads * vdim)
+    dot, top = denominator if denominator is not None else (None, None)
+    call("leone_head_norm_gate", _dev(o, "read-outs", torch.float32, (rows, heads * vdim)),
+         _dev(dot, "dot", torch.float32, (rows, heads)), _dev(top, "top", torch.float32, (rows, heads)),
+         _dev(gain, "gain"), _code(gain, "gain") if gain is not None else F32, per_head, gate_at, gate_stride,
+         ACTIVATIONS[activation], float(eps), _dev(out, "out"), _CODES[out_dtype], rows, heads, vdim, _stream())
+    return out
+
+
+def rms_mix(branches, gains, eps: float, scale: float) -> torch.Tensor:
+    """scale * sum_b rms(branches[b]) * gains[b]: every branch (float32 ``[rows, hidden]``) over its root mean
+    square along the row, times its gain."""
+    import ctypes
+    rows, hidden = branches[0].shape
+    if len(branches) != len(gains) or len({g.dtype for g in gains}) != 1:
+        raise KernelError("rms_mix: one gain a branch, all of one type")
+    out = torch.empty((rows, hidden), dtype=torch.float32, device=branches[0].device)
+    row_ptrs = (ctypes.c_void_p * len(branches))(*[_dev(b, "branch", torch.float32, (rows, hidden)) for b in branches])
+    gain_ptrs = (ctypes.c_void_p * len(gains))(*[_dev(g, "branch gain", None, (hidden,)) for g in gains])
+    call("leone_rms_mix", ctypes.cast(row_ptrs, ctypes.c_void_p), ctypes.cast(gain_ptrs, ctypes.c_void_p),
+         _code(gains[0], "branch gain"), len(branches), float(eps), float(scale), _dev(out, "out"), rows, hidden, _stream())
+    return out
+
+
+def relu_squared(x: torch.Tensor) -> torch.Tensor:
+    """max(x, 0)^2."""
+    out = torch.empty_like(x)
+    call("leone_relu_squared", _dev(x, "values"), _dev(out, "out"), _code(x, "values"), x.numel(), _stream())
+    return out
+
+
+def head_gate(out: torch.Tensor, gate: torch.Tensor, heads: int, vdim: int) -> torch.Tensor:
+    """out[r, h, :] *= sigmoid(gate[r, h]) in place; ``gate`` float32, possibly a slice of wider rows."""
+    rows = out.shape[0]
+    gate_at, gate_stride = _strided_rows(gate, "head gate", rows, heads)
+    call("leone_head_gate", _dev(out, "values", None, (rows, heads * vdim)), _code(out, "values"), gate_at, gate_stride,
+         rows, heads, vdim, _stream())
+    return out
+
+
+def scan_max_dim() -> int:
+    return int(library().leone_scan_max_dim())
+
+
+def outer_scan(proj: torch.Tensor, columns: dict, state: torch.Tensor, step, heads: int, dim: int, vdim: int, *,
+               gates: Optional[dict] = None, decay: Optional[torch.Tensor] = None, q_scale: float = 1.0,
+               k_scale: float = 1.0, cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+               write_state: bool = True):
+    """The matrix-memory recurrence S_t = a_t S_(t-1) + b_t k_t v_t^T, o_t = S_t^T q_t over every entry's rows,
+    from and into ``state`` (float32 ``[slots, heads, dim * vdim]``, with ``gates`` ``dim * vdim + dim + 1``: the
+    normaliser and the running maximum ride along).  ``proj`` is float32 ``[rows, width]``; ``columns`` names the
+    first column of q, k and v (and, with ``gates``, of the input and forget gates' pre-activations "i", "f").
+    ``gates`` = {"i_bias", "f_bias", "cap"}: exponential gates with a running maximum that starts at 0; else
+    ``decay`` (float32 ``[heads]``) with b = 1.  ``cos``/``sin``: rotary tables for q and k.
+    Returns o float32 ``[rows, heads * vdim]`` and, with gates, (dot, top) for ``head_norm_gate``."""
+    rows, width = proj.shape
+    per_head = dim * vdim + (dim + 1 if gates else 0)
+    if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (heads, per_head):
+        raise KernelError(f"outer_scan: state {tuple(state.shape)} is not [slots, {heads}, {per_head}] float32")
+    spans = entry_spans(step)
+    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=proj.device)
+    dot = top = None
+    if gates:
+        dot = torch.empty((rows, heads), dtype=torch.float32, device=proj.device)
+        top = torch.empty((rows, heads), dtype=torch.float32, device=proj.device)
+        if gates["i_bias"].dtype != gates["f_bias"].dtype:
+            raise KernelError("outer_scan: the gates' biases must share one type")
+    rotary_dim = 2 * cos.shape[1] if cos is not None else 0
+    call("leone_outer_scan", _dev(proj, "projection", torch.float32), width, columns["q"], columns["k"], columns["v"],
+         columns["i"] if gates else -1, columns["f"] if gates else -1,
+         _dev(gates["i_bias"], "i bias", None, (heads,)) if gates else 0,
+         _dev(gates["f_bias"], "f bias", None, (heads,)) if gates else 0,
+         _code(gates["i_bias"], "i bias") if gates else F32, float(gates["cap"]) if gates else 0.0,
+         _dev(decay, "decay", torch.float32, (heads,)) if decay is not None else 0, float(q_scale), float(k_scale),
+         _dev(cos, "rope cos", torch.float32), _dev(sin, "rope sin", torch.float32), rotary_dim,
+         cos.shape[0] if cos is not None else 0, _dev(state, "state"), state.stride(0), 1 if write_state else 0,
+         _dev(spans, "spans"), _dev(step.entry_slots, "slots", torch.int32),
+         _dev(step.positions, "positions", torch.int32, (rows,)), spans.shape[0], _dev(out, "out"),
+         _dev(dot, "dot"), _dev(top, "top"), heads, dim, vdim, _stream())
+    return (out, (dot, top)) if gates else (out, None)
+
+
+def delta_scan(qkv: torch.Tensor, columns: dict, beta: torch.Tensor, step_size: torch.Tensor, rate_log: torch.Tensor,
+               step_bias: torch.Tensor, state: torch.Tensor, step, heads: int, kv_heads: int, dim: int, vdim: int,
+               q_scale: float, unit_eps: float, write_state: bool = True) -> torch.Tensor:
+    """The gated delta rule over every entry's rows: S <- g * S with g = exp(-exp(rate_log) * softplus(step_size +
+    step_bias)) per head and key channel, u = sigmoid(beta) (v - S^T k), S <- S + k u^T, o = S^T q, with q and k
+    made unit vectors per head (x / sqrt(sum x^2 + unit_eps)) and q times ``q_scale``.  ``qkv`` float32 rows
+    holding q and k (``kv_heads`` heads of ``dim``) and v (``heads`` of ``vdim``) at ``columns``; ``beta`` float32
+    ``[rows, heads]`` and ``step_size`` ``[rows, heads * dim]`` may be slices of wider rows.  ``state`` float32
+    ``[slots, heads, dim, vdim]``.  Returns o float32 ``[rows, heads * vdim]``."""
+    rows = qkv.shape[0]
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, dim, vdim):
+        raise KernelError(f"delta_scan: state {tuple(state.shape)} is not [slots, {heads}, {dim}, {vdim}] float32")
+    if rate_log.dtype != step_bias.dtype:
+        raise KernelError("delta_scan: rate and step bias must share one type")
+    spans = entry_spans(step)
+    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=qkv.device)
+    beta_at, beta_stride = _strided_rows(beta, "delta_scan beta", rows, heads)
+    step_at, step_stride = _strided_rows(step_size, "delta_scan step", rows, heads * dim)
+    call("leone_delta_scan", _dev(qkv, "q, k, v", torch.float32), qkv.shape[1], columns["q"], columns["k"], columns["v"],
+         beta_at, beta_stride, step_at, step_stride, _dev(rate_log, "rate", None, (heads,)),
+         _dev(step_bias, "step bias", None, (heads * dim,)), _code(rate_log, "rate"), float(q_scale), float(unit_eps),
+         _dev(state, "state"), state.stride(0), 1 if write_state else 0, _dev(spans, "spans"),
+         _dev(step.entry_slots, "slots", torch.int32), _dev(step.positions, "positions", torch.int32, (rows,)),
+         spans.shape[0], _dev(out, "out"), heads, kv_heads, dim, vdim, _stream())
+    return out

@@ -28,9 +28,9 @@ _PROTOTYPES = {
     "leone_swiglu": [P, P, c_int, c_int, c_int, P],
     "leone_rope_table": [P, P, c_double, c_int, c_int, P],
     "leone_qk_norm_rope_write": [P, c_int, c_int, ctypes.c_long, P, P, P, c_int, P, P, c_int, c_float, P, P, c_int, c_int, c_int,
-                                 P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
-    "leone_attention_rows": [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
-                             c_int, P],
+                                 P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, ctypes.c_long, P],
+    "leone_attention_rows": [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                             c_int, P, ctypes.c_long, P],
     "leone_attention_decode_projected": [P, c_int, c_int, ctypes.c_long, P, P, c_int, c_float, P, P, c_int, c_int, c_int, P, P, P, c_int,
                                          P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, P],
     "leone_attention_decode": [P, P, P, P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
@@ -52,6 +52,18 @@ _PROTOTYPES = {
     "leone_sample_temperature": [P, P, P, P, P, P, P, P, c_int, c_int, P],
     "leone_top_candidates": [P, P, P, P, c_int, c_int, c_int, P],
     "leone_sample_truncated": [P, P, P, c_int, c_int, P],
+    "leone_add_layernorm": [P, P, P, P, c_float, P, P, c_int, c_float, P, c_int, P, c_int, c_int, P],
+    "leone_entry_spans": [P, c_int, P, P],
+    "leone_causal_conv": [P, c_int, ctypes.c_long, P, c_int, ctypes.c_long, P, c_int, P, c_int, P, c_int, P, P, P, c_int,
+                          c_int, c_int, c_int, c_int, P],
+    "leone_head_norm_gate": [P, P, P, P, c_int, c_int, P, ctypes.c_long, c_int, c_float, P, c_int, c_int, c_int, c_int, P],
+    "leone_rms_mix": [P, P, c_int, c_int, c_float, c_float, P, c_int, c_int, P],
+    "leone_relu_squared": [P, P, c_int, ctypes.c_long, P],
+    "leone_head_gate": [P, c_int, P, ctypes.c_long, c_int, c_int, c_int, P],
+    "leone_outer_scan": [P, ctypes.c_long, c_int, c_int, c_int, c_int, c_int, P, P, c_int, c_float, P, c_float, c_float,
+                         P, P, c_int, c_int, P, ctypes.c_long, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, P],
+    "leone_delta_scan": [P, ctypes.c_long, c_int, c_int, c_int, P, ctypes.c_long, P, ctypes.c_long, P, P, c_int, c_float,
+                         c_float, P, ctypes.c_long, c_int, P, P, P, c_int, P, c_int, c_int, c_int, c_int, P],
 }
 
 
@@ -83,6 +95,8 @@ def library() -> ctypes.CDLL:
             lib.leone_sample_truncated_params.argtypes = []
             lib.leone_peak_mfma_flops.restype = ctypes.c_double
             lib.leone_peak_mfma_flops.argtypes = [c_int, c_int]
+            lib.leone_scan_max_dim.restype = c_int
+            lib.leone_scan_max_dim.argtypes = []
             lib.leone_gemm_rows_max_rows.restype = c_int
             lib.leone_gemm_rows_max_rows.argtypes = []
             lib.leone_gemm_rows_chunk.restype = c_int

@@ -13,7 +13,8 @@ norm          ``tensor_specs()``, ``bind(tensors)``, ``add_norm(x, delta, out_dt
 position      ``prepare(max_positions, device)``; what it exposes to a mixer is
               the position part's own affair (the rotary part exposes tables).
 mixer         ``tensor_specs()``, ``bind(tensors)``, ``cache_need()`` -> ``KvNeed`` /
-              ``StateNeed`` / ``None``, ``forward(y, step, cache)`` -> delta ``[rows, hidden]``.
+              ``StateNeed`` / ``None``, or a dict name -> need for a mixer that keeps several things (its
+              ``forward`` then receives a dict name -> view), ``forward(y, step, cache)`` -> delta ``[rows, hidden]``.
               Optional: ``row_tiling()`` -> ``RowTiling`` if it has a kernel that works on tiles of rows.
 feed_forward  ``tensor_specs()``, ``bind(tensors)``, ``forward(y, step)`` -> delta.
               A mixer or feed-forward that sets ``fused_io = True`` is instead called with
@@ -72,11 +73,12 @@ class PartSpec:
 @dataclass(frozen=True)
 class KvNeed:
     """A mixer that caches one key and one value vector per token and kv head, packed in runs of 8:
-    keys ``[pages, kv_heads, head_dim/8, page_tokens, 8]``, values ``[pages, kv_heads, page_tokens/8, head_dim, 8]``."""
+    keys ``[pages, kv_heads, head_dim/8, page_tokens, 8]``, values ``[pages, kv_heads, page_tokens/8, value_dim, 8]``."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None   # only the last `window` positions are ever read
     page_tokens: Optional[int] = None   # tokens a page of this group holds; None: the engine's choice
+    value_dim: Optional[int] = None     # size of a value vector; None: the keys' size
 
     paged = True
 
@@ -88,7 +90,8 @@ class KvNeed:
             raise ValueError(f"the cache packs runs of 8: head_dim {self.head_dim} and page_tokens "
                              f"{page_tokens} must be multiples of 8")
         return (torch.zeros((pages, self.kv_heads, self.head_dim // 8, page_tokens, 8), dtype=dtype, device=device),
-                torch.zeros((pages, self.kv_heads, page_tokens // 8, self.head_dim, 8), dtype=dtype, device=device))
+                torch.zeros((pages, self.kv_heads, page_tokens // 8, self.value_dim or self.head_dim, 8), dtype=dtype,
+                            device=device))
 
     def view(self, storage, block_table, page_tokens: int):
         from .context import KvCacheView
@@ -100,7 +103,7 @@ class KvNeed:
             pool.index_fill_(0, index, float("nan"))
 
     def bytes_per_token(self, element_size: int) -> int:
-        return 2 * self.kv_heads * self.head_dim * element_size
+        return self.kv_heads * (self.head_dim + (self.value_dim or self.head_dim)) * element_size
 
 
 @dataclass(frozen=True)
@@ -174,10 +177,31 @@ class Registry:
         return sorted(self._classes)
 
 
+def flatten_needs(need, path=()):
+    """A part may need several kinds of storage at once (a mixer with keys and a state, a block whose
+    sublayers keep their own inputs): it then answers ``cache_need()`` with a dict name -> need (or dict).
+    This lists the leaves as (path of names, need); a plain need is the one leaf ``((), need)``."""
+    if isinstance(need, dict):
+        found = []
+        for name, inner in need.items():
+            found += flatten_needs(inner, path + (name,))
+        return found
+    return [] if need is None else [(path, need)]
+
+
+def nest_views(need, path, lookup):
+    """The views of a part's needs in the shape of the needs: a dict name -> view (or dict) for a dict of needs,
+    the view itself for a plain need.  ``lookup(path)`` gives the view of a leaf."""
+    if isinstance(need, dict):
+        return {name: nest_views(inner, path + (name,), lookup) for name, inner in need.items()}
+    return None if need is None else lookup(path)
+
+
 NORMS = Registry("norm")
 POSITIONS = Registry("position")
 MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed_forward")
+CONVS = Registry("conv")
 BLOCKS = Registry("block")
 
 

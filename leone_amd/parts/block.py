@@ -6,7 +6,8 @@ from typing import Dict, List, Optional
 import torch
 
 from ..weights.loader import TensorSpec
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Part, PartSpec
+from .. import ops
+from .base import BLOCKS, CONVS, FEED_FORWARDS, MIXERS, NORMS, Part, PartSpec
 from .context import CacheView, StepContext
 
 
@@ -86,3 +87,85 @@ class PreNormBlock(Part):
         if getattr(consumer, "fused_io", False) and hasattr(norm, "lazy"):
             return norm.lazy(x, delta, step.dtype)
         return norm.add_norm(x, delta, step.dtype)
+
+
+@BLOCKS.register("sandwich")
+class SandwichBlock(Part):
+    """A norm before and one behind each sublayer, and a short causal convolution on what a sublayer reads:
+
+        x <- x + norm1b(mixer(conv1(norm1(x))));   x <- x + norm2b(feed_forward(conv2(norm2(x))))
+
+    The second sublayer is there only if ``feed_forward`` is given; a ``conv`` may be None (the sublayer reads
+    the norm's result as it is).  The convolutions keep their last inputs per request, so the block's cache need
+    is a dict: ``mixer`` (the mixer's own), ``conv1``, ``conv2``.
+
+    Parameters: ``norm1``, ``conv1``, ``mixer``, ``norm1b`` and optionally ``norm2``, ``conv2``,
+    ``feed_forward``, ``norm2b`` (part specs).  The norm behind a sublayer is not carried out here: the block
+    hands on ``ops.NormedDelta`` and the norm that runs next does it together with the residual sum and its own.
+    """
+
+    def __init__(self, spec: PartSpec, **context):
+        def optional(registry, key):
+            return registry.build(spec[key], **context) if spec.get(key) is not None else None
+        self.norm1 = NORMS.build(spec["norm1"], **context)
+        self.conv1 = optional(CONVS, "conv1")
+        self.mixer = MIXERS.build(spec["mixer"], **context)
+        self.norm1b = NORMS.build(spec["norm1b"], **context)
+        self.feed_forward = optional(FEED_FORWARDS, "feed_forward")
+        self.norm2 = optional(NORMS, "norm2")
+        self.conv2 = optional(CONVS, "conv2")
+        self.norm2b = optional(NORMS, "norm2b")
+        if self.feed_forward is not None and (self.norm2 is None or self.norm2b is None):
+            raise ValueError("a sandwich block with a feed-forward needs norm2 and norm2b")
+
+    def parts(self):
+        return tuple(part for part in (self.norm1, self.conv1, self.mixer, self.norm1b, self.norm2, self.conv2,
+                                       self.feed_forward, self.norm2b) if part is not None)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", False) for part in self.parts())
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for part in self.parts() for s in part.tensor_specs()]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for part in self.parts():
+            part.bind(tensors)
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [w for part in self.parts() if hasattr(part, "streamed_weights") for w in part.streamed_weights()]
+
+    def cache_need(self):
+        need = {"mixer": self.mixer.cache_need()}
+        if self.conv1 is not None:
+            need["conv1"] = self.conv1.cache_need()
+        if self.conv2 is not None and self.feed_forward is not None:
+            need["conv2"] = self.conv2.cache_need()
+        return need
+
+    def row_tilings(self):
+        found = []
+        for part in self.parts():
+            if hasattr(part, "row_tiling"):
+                found.append(part.row_tiling())
+            if hasattr(part, "row_tilings"):
+                found += part.row_tilings()
+        return found
+
+    @staticmethod
+    def _read(norm, conv, x, pending, step, cache):
+        """What a sublayer reads: the norm of the stream (which first takes in what is pending), through the
+        convolution if there is one."""
+        if conv is None:
+            return norm.add_norm(x, pending, step.dtype)
+        return conv.forward(norm.add_norm(x, pending, torch.float32), step, cache, step.dtype)
+
+    def forward(self, x: torch.Tensor, pending, step: StepContext, cache):
+        cache = cache or {}
+        h = self._read(self.norm1, self.conv1, x, pending, step, cache.get("conv1"))
+        pending = ops.NormedDelta(self.mixer.forward(h, step, cache.get("mixer")), self.norm1b)
+        if self.feed_forward is None:
+            return pending
+        h = self._read(self.norm2, self.conv2, x, pending, step, cache.get("conv2"))
+        return ops.NormedDelta(self.feed_forward.forward(h, step), self.norm2b)

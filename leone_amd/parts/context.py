@@ -48,6 +48,8 @@ class StepContext:
     # Long portions come first in a step.  For every tiling a part of the model declared (``RowTiling``) that
     # cuts at least one portion of this step: the tile list and the rows it covers.
     tiled: Dict[object, TiledRows] = field(default_factory=dict)
+    # int32 [entries, 2] on the device: first row and end of every entry (``ops.entry_spans`` makes it on first use).
+    spans: Optional[torch.Tensor] = None
 
 
 @dataclass

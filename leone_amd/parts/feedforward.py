@@ -58,3 +58,30 @@ class SwiGluMlp(Part):
         and with ``next_norm`` the norm that follows may come back prepared (see ``ops.linear``)."""
         activated = ops.linear(y, self.w_gate_up, gated=True)
         return ops.linear(activated, self.w_down, residual=residual, next_norm=next_norm)
+
+
+@FEED_FORWARDS.register("relu2")
+class ReluSquaredMlp(Part):
+    """down(relu(up y)^2), no bias.  Parameters: ``hidden``, ``intermediate`` and tensor names ``up``, ``down``."""
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, **_):
+        p = spec.params
+        self.hidden, self.intermediate = int(p["hidden"]), int(p["intermediate"])
+        self.names = {k: p[k] for k in ("up", "down")}
+        self.w_up = self.w_down = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.names["up"], (self.intermediate, self.hidden), MATRIX),
+                TensorSpec(self.names["down"], (self.hidden, self.intermediate), MATRIX)]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.w_up = tensors.pop(self.names["up"]).contiguous()
+        self.w_down = tensors.pop(self.names["down"]).contiguous()
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.w_up, self.w_down]
+
+    def forward(self, y: torch.Tensor, step: StepContext) -> torch.Tensor:
+        return ops.linear(ops.relu_squared(ops.linear(y, self.w_up)), self.w_down, out_dtype=torch.float32)

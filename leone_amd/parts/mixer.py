@@ -28,6 +28,10 @@ class GqaAttention(Part):
     Parameters: ``hidden``, ``q_heads``, ``kv_heads``, ``head_dim``, ``qk_norm_eps``
     (None: no q/k norm), ``window`` (None: all keys), ``position`` (name of a
     position part) and tensor names ``q``, ``k``, ``v``, ``o``, ``q_norm``, ``k_norm``.
+    Optional: ``scale`` (the scores' factor, 1/sqrt(head_dim) if absent), ``value_dim`` (values and the output
+    of a head have this size instead of ``head_dim``), ``gate`` (tensor name ``[q_heads, hidden]``: head h's
+    result is multiplied by sigmoid(gate y)_h before the output projection), ``float_output`` (the output
+    projection's result comes in float32 whatever the engine's type).
     """
 
     graph_safe = True
@@ -44,6 +48,12 @@ class GqaAttention(Part):
         self.window = p.get("window")
         self.scale = float(p.get("scale", 1.0 / math.sqrt(self.head_dim)))
         self.names = {k: p[k] for k in ("q", "k", "v", "o")}
+        self.value_dim = int(p.get("value_dim") or self.head_dim)
+        self.float_output = bool(p.get("float_output", False))
+        if p.get("gate"):
+            self.names["gate"] = p["gate"]
+        # a value size of its own or a gate: the projection carries more than q, k and v of one size
+        self.general = self.value_dim != self.head_dim or "gate" in self.names
         if self.qk_norm_eps is not None:
             self.names.update(q_norm=p["q_norm"], k_norm=p["k_norm"])
         self.position = (positions or {}).get(p.get("position")) if p.get("position") else None
@@ -52,7 +62,8 @@ class GqaAttention(Part):
         self.w_qkv = self.w_o = self.q_gain = self.k_gain = None
 
     def cache_need(self) -> KvNeed:
-        return KvNeed(self.kv_heads, self.head_dim, self.window)
+        return KvNeed(self.kv_heads, self.head_dim, self.window,
+                      value_dim=self.value_dim if self.value_dim != self.head_dim else None)
 
     def row_tiling(self) -> RowTiling:
         """The tiles of the prompt-attention kernel."""
@@ -62,8 +73,10 @@ class GqaAttention(Part):
         qw, kvw = self.q_heads * self.head_dim, self.kv_heads * self.head_dim
         specs = [TensorSpec(self.names["q"], (qw, self.hidden), MATRIX),
                  TensorSpec(self.names["k"], (kvw, self.hidden), MATRIX),
-                 TensorSpec(self.names["v"], (kvw, self.hidden), MATRIX),
-                 TensorSpec(self.names["o"], (self.hidden, qw), MATRIX)]
+                 TensorSpec(self.names["v"], (self.kv_heads * self.value_dim, self.hidden), MATRIX),
+                 TensorSpec(self.names["o"], (self.hidden, self.q_heads * self.value_dim), MATRIX)]
+        if "gate" in self.names:
+            specs.append(TensorSpec(self.names["gate"], (self.q_heads, self.hidden), MATRIX))
         if self.qk_norm_eps is not None:
             specs += [TensorSpec(self.names["q_norm"], (self.head_dim,), VECTOR),
                       TensorSpec(self.names["k_norm"], (self.head_dim,), VECTOR)]
@@ -71,8 +84,10 @@ class GqaAttention(Part):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         # One product for q, k and v: a pure re-layout of the three matrices.
-        self.w_qkv = torch.cat([tensors.pop(self.names["q"]), tensors.pop(self.names["k"]),
-                                tensors.pop(self.names["v"])], dim=0).contiguous()
+        fused = [tensors.pop(self.names["q"]), tensors.pop(self.names["k"]), tensors.pop(self.names["v"])]
+        if "gate" in self.names:
+            fused.append(tensors.pop(self.names["gate"]))      # the heads' gates ride along as further columns
+        self.w_qkv = torch.cat(fused, dim=0).contiguous()
         self.w_o = tensors.pop(self.names["o"]).contiguous()
         if self.qk_norm_eps is not None:
             self.q_gain = tensors.pop(self.names["q_norm"]).contiguous()
@@ -90,6 +105,22 @@ class GqaAttention(Part):
                 residual: Optional[torch.Tensor] = None, next_norm=None):
         """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned),
         and with ``next_norm`` the norm that follows may come back prepared (see ``ops.linear``)."""
+        out_dtype = torch.float32 if self.float_output else None
+        rotation = rotation_of(self.position)
+        if rotation.cos is not None and step.max_position >= rotation.cos.shape[0]:
+            raise ValueError(f"position {step.max_position} is beyond the rotary table of {rotation.cos.shape[0]} positions")
+        if self.general:
+            proj = ops.linear(y, self.w_qkv, out_dtype=torch.float32)
+            q = ops.qk_norm_rope_write(proj, self.q_heads, self.kv_heads, self.head_dim, self.q_gain, self.k_gain,
+                                       self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, rotation.cos, rotation.sin,
+                                       step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
+                                       write_cache=cache.writes, out_dtype=step.dtype, pairing=rotation.pairing,
+                                       value_dim=self.value_dim)
+            gate = None
+            if "gate" in self.names:
+                gate = proj[:, (self.q_heads + self.kv_heads) * self.head_dim + self.kv_heads * self.value_dim:]
+            attended = self._attend(q, step, cache, gate)
+            return ops.linear(attended, self.w_o, out_dtype=out_dtype, residual=residual, next_norm=next_norm)
         qkv = ops.linear(y, self.w_qkv, planes_ok=True)
         # How much of a head is rotated and in which pairs is the position part's affair; the kernels are told.
         rotation = rotation_of(self.position)
@@ -104,13 +135,13 @@ class GqaAttention(Part):
                 self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin, cache.k_pool, cache.v_pool,
                 step.positions, step.row_entry, cache.block_table, self.scale, int(self.window or 0),
                 max_context=step.max_position + 1, write_cache=cache.writes, pairing=rotation.pairing)
-            return ops.linear(attended, self.w_o, residual=residual, next_norm=next_norm)
+            return ops.linear(attended, self.w_o, out_dtype=out_dtype, residual=residual, next_norm=next_norm)
         q = ops.qk_norm_rope_write(qkv, self.q_heads, self.kv_heads, self.head_dim, self.q_gain, self.k_gain,
                                    self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin,
                                    step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
                                    write_cache=cache.writes, out_dtype=step.dtype, pairing=rotation.pairing)
         attended = self._attend(q, step, cache)
-        return ops.linear(attended, self.w_o, residual=residual, next_norm=next_norm)
+        return ops.linear(attended, self.w_o, out_dtype=out_dtype, residual=residual, next_norm=next_norm)
 
     def attention_kernels(self, dtype: torch.dtype, page_tokens: int, max_blocks: int = 0) -> Dict[str, str]:
         """Which kernels this shape gets, by kind of work: ``decode`` (steps of single tokens): "projected" (the
@@ -119,22 +150,24 @@ class GqaAttention(Part):
         ``prompt`` (portions of at least ``ops.PREFILL_MIN_ROWS`` rows): "flash" (the matrix-core prompt
         kernel), else what single tokens get."""
         group = self.q_heads // self.kv_heads
-        if not ops.decode_attention_supported(dtype, self.head_dim, page_tokens, group, max_blocks):
+        if self.value_dim != self.head_dim or not ops.decode_attention_supported(dtype, self.head_dim, page_tokens, group, max_blocks):
             return {"decode": "rows", "prompt": "rows"}
         rotation = rotation_of(self.position)
-        projected = ops.decode_projected_supported(self.head_dim, rotation.rotary_dim, rotation.pairing)
+        projected = not self.general and ops.decode_projected_supported(self.head_dim, rotation.rotary_dim, rotation.pairing)
         return {"decode": "projected" if projected else "split_kv",
                 "prompt": "flash" if ops.prefill_attention_supported(dtype, self.head_dim, page_tokens, max_blocks) else "split_kv"}
 
-    def _attend(self, q: torch.Tensor, step: StepContext, cache: KvCacheView) -> torch.Tensor:
+    def _attend(self, q: torch.Tensor, step: StepContext, cache: KvCacheView, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Long prompt portions through the prompt kernel, the other rows through the split-KV kernel; the
-        row kernel takes what the matrix-core kernels refuse (float32, odd sizes)."""
+        row kernel takes what the matrix-core kernels refuse (float32, odd sizes, values of another size than
+        the keys).  ``gate``: the heads' gates (float32 ``[rows, q_heads]``), applied to the result."""
         window = int(self.window or 0)
         group = self.q_heads // self.kv_heads
         max_blocks = cache.block_table.shape[1]
-        if not ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens, group, max_blocks):
+        if self.value_dim != self.head_dim or \
+                not ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens, group, max_blocks):
             return ops.attention_rows(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
-                                      cache.block_table, self.q_heads, self.scale, window)
+                                      cache.block_table, self.q_heads, self.scale, window, gate=gate)
         first = 0
         out = torch.empty_like(q)
         tiled = step.tiled.get(self.row_tiling())
@@ -148,4 +181,4 @@ class GqaAttention(Part):
             ops.attention_decode(q[first:], cache.k_pool, cache.v_pool, step.positions[first:],
                                  step.row_entry[first:], cache.block_table, self.q_heads, self.scale, window,
                                  max_context=step.max_position + 1, out=out[first:])
-        return out
+        return out if gate is None else ops.head_gate(out, gate, self.q_heads, self.value_dim)

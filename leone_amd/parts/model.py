@@ -8,7 +8,7 @@ import torch
 
 from .. import ops
 from ..weights.loader import MATRIX, TensorSpec
-from .base import BLOCKS, NORMS, POSITIONS, PartSpec
+from .base import BLOCKS, NORMS, POSITIONS, PartSpec, flatten_needs, nest_views
 from .context import CacheView, StepContext
 
 
@@ -176,25 +176,48 @@ class DecoderModel:
 
     # ---- cache ---------------------------------------------------------------
     def cache_needs(self) -> Dict[int, object]:
-        """Cache slot -> what the layer runs on it need (one need per slot)."""
-        needs: Dict[int, object] = {}
-        writers: Dict[int, int] = {}
+        """Cache slot -> what the layer runs on it need (one need per slot).  A layer that needs several kinds
+        of storage (``cache_need()`` answers with a dict, see ``parts.base.flatten_needs``) gets one slot for
+        each, keyed (the run's slot, *names)."""
+        needs: Dict[object, object] = {}
+        writers: Dict[object, int] = {}
         for run in self.schedule:
             need = self.layers[run.layer].cache_need()
-            if need is None:
+            leaves = flatten_needs(need)
+            if not leaves:
                 if run.cache is not None:
                     raise ValueError(f"layer {run.layer} keeps no cache but its run names slot {run.cache}")
                 continue
             if run.cache is None:
                 raise ValueError(f"layer {run.layer} needs a cache but its run names none")
-            if run.cache in needs and needs[run.cache] != need:
-                raise ValueError(f"cache slot {run.cache} is shared by layers with different needs")
-            needs[run.cache] = need
+            for path, leaf in leaves:
+                key = (run.cache,) + path if isinstance(need, dict) else run.cache
+                if key in needs and needs[key] != leaf:
+                    raise ValueError(f"cache slot {key} is shared by layers with different needs")
+                needs[key] = leaf
             writers[run.cache] = writers.get(run.cache, 0) + (1 if run.writes else 0)
         for slot, count in writers.items():
             if count != 1:
                 raise ValueError(f"cache slot {slot} must have exactly one writing run, found {count}")
         return needs
+
+    @staticmethod
+    def _cache_of(run: LayerRun, layer, caches: Dict[object, CacheView]):
+        """What a run's layer receives as its cache: the view of the run's slot, or, for a layer with several
+        needs, the views in the shape of its needs."""
+        if run.cache is None:
+            return None
+
+        def view(key):
+            found = caches.get(key)
+            if found is not None and found.writes != run.writes:
+                found = type(found)(**{**found.__dict__, "writes": run.writes})
+            return found
+
+        need = layer.cache_need()
+        if isinstance(need, dict):
+            return nest_views(need, (run.cache,), view)
+        return view(run.cache)
 
     # ---- forward ---------------------------------------------------------------
     def forward(self, tokens: torch.Tensor, step: StepContext, caches: Dict[int, CacheView]) -> Optional[torch.Tensor]:
@@ -202,10 +225,8 @@ class DecoderModel:
         x = ops.embed(self.embedding, tokens, scale=self.spec.embedding_scale or 1.0)
         pending = None
         for at, run in enumerate(self.schedule):
-            cache = caches.get(run.cache) if run.cache is not None else None
-            if cache is not None and cache.writes != run.writes:
-                cache = type(cache)(**{**cache.__dict__, "writes": run.writes})
             layer = self.layers[run.layer]
+            cache = self._cache_of(run, layer, caches)
             # A block that can do so leaves the first norm of the block that runs next prepared.
             after = self.layers[self.schedule[at + 1].layer] if at + 1 < len(self.schedule) else None
             next_norm = after.entry_norm(step.dtype) if hasattr(after, "entry_norm") else None

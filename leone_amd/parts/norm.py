@@ -35,6 +35,8 @@ class RmsNorm(Part):
                  rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         if isinstance(delta, ops.PreparedRows):
             delta = None                      # the product that made it has added into the stream already
+        if isinstance(delta, ops.NormedDelta):
+            delta = delta.materialize()       # a delta that another kind of norm is still to be applied to
         return ops.add_rmsnorm(x, delta, self.gain, self.eps, out_dtype, rows)
 
     def folded(self, out_dtype: torch.dtype):
@@ -53,3 +55,49 @@ class RmsNorm(Part):
         if delta is not None:
             return self.add_norm(x, delta, out_dtype, rows)
         return ops.NormedRows(x, self.gain, self.eps, out_dtype, rows)
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Part):
+    """y = (x - mean) / sqrt(var + eps) * weight + bias, var the mean squared deviation; mean and variance in float.
+
+    Parameters: ``size``, ``eps``, ``weight``, ``bias`` (tensor names).  ``add_norm`` also takes a delta that
+    is still to go through another layer norm (``ops.NormedDelta``: the norm behind a sublayer) and does that
+    norm, the residual sum and its own in one kernel.
+    """
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, **_):
+        self.size = int(spec["size"])
+        self.eps = float(spec["eps"])
+        self.weight_name, self.bias_name = spec["weight"], spec["bias"]
+        self.gain: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.weight_name, (self.size,), VECTOR), TensorSpec(self.bias_name, (self.size,), VECTOR)]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.gain = tensors[self.weight_name].contiguous()
+        self.bias = tensors[self.bias_name].contiguous()
+        if self.gain.dtype != self.bias.dtype:
+            self.gain, self.bias = self.gain.float(), self.bias.float()
+
+    def add_norm(self, x: torch.Tensor, delta, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if isinstance(delta, ops.PreparedRows):
+            delta = None
+        delta_norm = None
+        if isinstance(delta, ops.NormedDelta):
+            behind = delta.norm
+            if isinstance(behind, LayerNorm) and behind.gain.dtype == self.gain.dtype:
+                delta, delta_norm = delta.rows, (behind.gain, behind.bias, behind.eps)
+            else:
+                delta = delta.materialize()
+        elif delta is not None and delta.dim() == 3:
+            delta = delta.sum(dim=0)          # planes of a product cut along its inner dimension
+        return ops.add_layernorm(x, delta, self.gain, self.bias, self.eps, out_dtype, rows, delta_norm)
+
+    def apply(self, rows: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        """The norm of float32 rows that are no stream (nothing is added, nothing written back)."""
+        return ops.add_layernorm(rows, None, self.gain, self.bias, self.eps, out_dtype)
