@@ -1,0 +1,441 @@
+"""Pamevik on the GPU against the plain implementation: each mechanism alone, whole models of several sizes under
+every way of cutting the work, state slots and pages that are used again, long decoding, and generation through
+the scheduler."""
+import json
+import math
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests import pamevik_util as pu
+from tests import schedules
+from tests.plain import pamevik_plain as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+# float32: sums of a few hundred float products; bfloat16: 8 significant bits wherever an activation is stored.
+# Measured: float32 2e-7 to 3e-6, bfloat16 3e-3 to 1.2e-2 of the logits' size.
+TOLERANCE = {"float32": 3e-5, "bfloat16": 4e-2}
+LENGTHS = {"P": [1, 2, 37, 130, 64, 9], "Q": [70, 3, 150, 33, 81], "R": [90, 17, 65, 2, 48], "S": [5, 100, 31, 66, 12]}
+
+
+def widened(weights):
+    return {k: v.float() if v.is_floating_point() else v for k, v in weights.items()}
+
+
+@pytest.fixture(scope="module")
+def cases(tmp_path_factory):
+    cache = {}
+
+    def get(name, dtype_name):
+        key = (name, dtype_name)
+        if key not in cache:
+            raw = pu.SMALL[name]
+            weights = pu.make_weights(raw, 17 + len(cache), pu.RANKS[name], DTYPES[dtype_name],
+                                      sharpen=3.0 if dtype_name == "float32" else 1.0)
+            folder = pu.write_dir(str(tmp_path_factory.mktemp(f"pamevik_{name}_{dtype_name}")), raw, weights)
+            gen = np.random.default_rng(5 + len(cache))
+            requests = {f"r{i}": gen.integers(0, raw["vocab"], size=n).tolist() for i, n in enumerate(LENGTHS[name])}
+            expected = {rid: plain.forward(raw, widened(weights), toks).numpy() for rid, toks in requests.items()}
+            cache[key] = (folder, requests, expected)
+        return cache[key]
+    return get
+
+
+def make_engine(folder, dtype_name, **options):
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+    options.setdefault("page_tokens", 16)
+    options.setdefault("max_requests", 4)
+    return Engine(load_model(folder, dtype_name), **options)
+
+
+def run_steps(engine, steps):
+    from leone_amd.engine.engine import StepEntry
+    outputs = {}
+    for s in steps:
+        out = engine.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        if out.logits is not None:
+            outputs[s["step"]] = out.logits.float().cpu().numpy()
+        for rid in s["end"]:
+            engine.release(rid)
+        engine.cache.check()
+    return outputs
+
+
+def compare(steps, outputs, expected, tol, what):
+    got = schedules.collect(steps, outputs)
+    assert set(got) == set(expected)
+    worst_seen = 0.0
+    for rid, rows in got.items():
+        have, want = np.stack(rows), expected[rid]
+        assert have.shape == want.shape and np.isfinite(have).all(), (what, rid, have.shape, want.shape)
+        err = pu.relative_error(have, want)
+        worst_seen = max(worst_seen, float(err.max()))
+        assert err.max() <= tol, (f"{what}: request {rid} first wrong position {int(np.argmax(err > tol))} of {len(err)}, "
+                                  f"worst {int(err.argmax())}: {err.max():.3e} > {tol}")
+    return worst_seen
+
+
+SCHEDULES = {"whole": schedules.whole, "tail_decoded": lambda r: schedules.tail_decoded(r, 20),
+             "portions": schedules.portions, "mixed": schedules.mixed}
+
+
+@pytest.mark.parametrize("schedule", list(SCHEDULES))
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+@pytest.mark.parametrize("name", list(pu.SMALL))
+def test_engine_agrees_with_plain_however_the_work_is_cut(cases, name, dtype_name, schedule):
+    """Whole prompts, tails decoded token by token, portions down to two tokens, and four requests at a time with
+    portions beside single tokens, on an engine with four state slots and just enough pages: slots and pages are
+    used again.  Logits at every position against the plain implementation."""
+    folder, requests, expected = cases(name, dtype_name)
+    steps = SCHEDULES[schedule](requests)
+    room = schedules.max_live_tokens(steps, 16)
+    engine = make_engine(folder, dtype_name, max_tokens=room)
+    outputs = run_steps(engine, steps)
+    worst = compare(steps, outputs, expected, TOLERANCE[dtype_name], f"{name} {dtype_name} {schedule}")
+    print(f"{name} {dtype_name} {schedule}: worst relative error {worst:.2e}")
+    assert all(engine.cache.free_pages(g) == engine.cache.groups[g].num_pages for g in range(len(engine.cache.groups)))
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_a_slot_that_held_another_request_starts_from_zero(cases, dtype_name):
+    """One state slot: every request runs where the one before it left its state, and what a freed slot holds is
+    overwritten with NaN here, as a fault would leave it.  Each request must come out as if it were alone."""
+    folder, requests, expected = cases("P", dtype_name)
+    engine = make_engine(folder, dtype_name, max_tokens=192, max_requests=1)
+    for rid, toks in requests.items():
+        steps = schedules.portions({rid: toks}, sizes=(3, 1, 2, 40))
+        outputs = run_steps(engine, steps)
+        compare(steps, outputs, {rid: expected[rid]}, TOLERANCE[dtype_name], f"slot reuse {rid}")
+        for storage in engine.pools.state.values():
+            storage.fill_(float("nan"))
+        for storage in engine.pools.paged.values():
+            for pool in storage:
+                pool.fill_(float("nan"))
+
+
+def test_long_decoding_through_recorded_steps(cases):
+    """A short prompt, then 300 tokens one by one (steps replayed from a recording), two requests side by side."""
+    raw = pu.SMALL["P"]
+    weights = pu.make_weights(raw, 91, pu.RANKS["P"], torch.float32)
+    gen = np.random.default_rng(2)
+    requests = {"a": gen.integers(0, raw["vocab"], size=310).tolist(), "b": gen.integers(0, raw["vocab"], size=305).tolist()}
+    expected = {rid: plain.forward(raw, weights, toks).numpy() for rid, toks in requests.items()}
+    import tempfile
+    with tempfile.TemporaryDirectory() as folder:
+        pu.write_dir(folder, raw, weights)
+        for graphs in (True, False):
+            engine = make_engine(folder, "float32", max_tokens=704, graphs=graphs)
+            steps = [{"step": 0, "entries": [{"id": "a", "tokens": requests["a"][:10], "want": list(range(10))},
+                                             {"id": "b", "tokens": requests["b"][:5], "want": list(range(5))}], "end": []}]
+            for i in range(300):
+                steps.append({"step": i + 1, "entries": [{"id": "a", "tokens": [requests["a"][10 + i]], "want": [0]},
+                                                         {"id": "b", "tokens": [requests["b"][5 + i]], "want": [0]}],
+                              "end": ["a", "b"] if i == 299 else []})
+            assert engine.graphs == graphs
+            outputs = run_steps(engine, steps)
+            compare(steps, outputs, expected, TOLERANCE["float32"], f"long decoding, graphs {graphs}")
+
+
+def test_greedy_generation_through_the_scheduler(cases):
+    """The framework's own entry point: prompts in, greedy tokens out, scheduled in portions with more requests
+    than state slots, against the plain implementation's argmax token by token."""
+    from leone_amd.api import Runtime
+    from leone_amd.engine.scheduler import SchedulerPolicy
+    raw = pu.SMALL["Q"]
+    weights = pu.make_weights(raw, 23, pu.RANKS["Q"], torch.float32)
+    gen = np.random.default_rng(8)
+    prompts = [gen.integers(0, raw["vocab"], size=n).tolist() for n in (3, 40, 21, 9, 57)]
+    import tempfile
+    with tempfile.TemporaryDirectory() as folder:
+        pu.write_dir(folder, raw, weights)
+        runtime = Runtime.load(folder, "float32", max_tokens=512, page_tokens=16, max_requests=2,
+                               policy=SchedulerPolicy(max_live_requests=2, prefill_chunk_tokens=16, max_step_tokens=24))
+        results = runtime.generate_tokens(prompts, 12, eos_token_id=None)
+    for prompt, result in zip(prompts, results):
+        tokens = list(prompt)
+        for i in range(12):
+            logits = plain.forward(raw, weights, tokens)[-1]
+            best = int(logits.argmax())
+            if result.tokens[i] != best:       # a near tie may fall either way; anything else is a fault
+                assert float(logits[best] - logits[result.tokens[i]]) < 1e-4, (i, best, result.tokens[i])
+            tokens.append(result.tokens[i])
+        assert len(result.tokens) == 12
+
+
+def test_trace_replay_as_a_user_runs_it(cases, tmp_path):
+    folder, requests, expected = cases("R", "float32")
+    steps = schedules.mixed(requests)
+    out_dir = str(tmp_path / "out")
+    process = subprocess.Popen([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                                "--out", out_dir, "--max-tokens", str(schedules.max_live_tokens(steps, 64))],
+                               stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    outputs = {}
+    for s in steps:
+        process.stdin.write(json.dumps(s) + "\n")
+        process.stdin.flush()
+        assert process.stdout.readline().strip() == f"done {s['step']}"
+        wanted = sum(len(e["want"]) for e in s["entries"])
+        if wanted:
+            outputs[s["step"]] = np.fromfile(os.path.join(out_dir, f"{s['step']}.f32"), dtype="<f4").reshape(wanted, -1)
+    process.stdin.close()
+    assert process.wait(timeout=60) == 0
+    compare(steps, outputs, expected, TOLERANCE["float32"], "trace replay")
+
+
+# ---- each mechanism alone ---------------------------------------------------------------------------------------
+
+def step_of(rows_meta, dtype, slots, tables=None):
+    """A StepContext for rows [(entry, position)] in order; entry e uses state slot slots[e]."""
+    from leone_amd.parts.context import StepContext
+    n_entries = max(e for e, _ in rows_meta) + 1
+    return StepContext(rows=len(rows_meta), dtype=dtype, device=torch.device(DEV),
+                       positions=torch.tensor([p for _, p in rows_meta], dtype=torch.int32, device=DEV),
+                       row_entry=torch.tensor([e for e, _ in rows_meta], dtype=torch.int32, device=DEV), entries=[],
+                       entry_slots=torch.tensor(slots[:n_entries], dtype=torch.int32, device=DEV), want_rows=None,
+                       block_tables=tables or {}, max_position=max(p for _, p in rows_meta))
+
+
+def views_of(need, slots=3, pages=40, page_tokens=16, dtype=torch.float32):
+    """Storage and views for a part's needs: state per slot filled with NaN (a request's first step must not read
+    it), pages likewise; every entry's block table lists its own pages in a scattered order."""
+    from leone_amd.parts.base import flatten_needs, nest_views
+    made = {}
+    for path, leaf in flatten_needs(need):
+        if leaf.paged:
+            storage = leaf.allocate(pages, page_tokens, dtype, DEV)
+            for pool in storage:
+                pool.fill_(float("nan"))
+            made[path] = ("paged", leaf, storage)
+        else:
+            storage = leaf.allocate_slots(slots, DEV)
+            storage.fill_(float("nan"))
+            made[path] = ("state", leaf, storage)
+    return made
+
+
+def nested(need, made, table):
+    from leone_amd.parts.base import nest_views
+    def view(path):
+        kind, leaf, storage = made[path]
+        return leaf.view(storage, table, 16) if kind == "paged" else leaf.view(storage)
+    return nest_views(need, (), view)
+
+
+def run_mixer_in_cuts(mixer, hs, cuts, dtype):
+    """Feeds two sequences (``hs``: [steps, width] each) to a mixer part in steps: ``cuts`` lists, per step, how
+    many rows of each sequence it brings (0: the sequence sits the step out).  Sequence 0 lives in state slot 2,
+    sequence 1 in slot 0; their pages are interleaved.  Returns each sequence's outputs in order."""
+    need = mixer.cache_need()
+    made = views_of(need, dtype=dtype)
+    pages = {0: list(range(1, 40, 2)), 1: list(range(0, 40, 2))}
+    at, outs = [0, 0], [[], []]
+    for cut in cuts:
+        present = [s for s in (0, 1) if cut[s]]
+        meta, rows = [], []
+        for e, s in enumerate(present):
+            meta += [(e, at[s] + i) for i in range(cut[s])]
+            rows.append(hs[s][at[s]:at[s] + cut[s]])
+        table = torch.tensor([pages[s] for s in present], dtype=torch.int32, device=DEV)
+        step = step_of(meta, dtype, [(2, 0)[s] for s in present], {0: table})
+        result = mixer.forward(torch.cat(rows).to(DEV).to(dtype), step, nested(need, made, table))
+        first = 0
+        for s in present:
+            outs[s].append(result[first:first + cut[s]].float().cpu())
+            first += cut[s]
+            at[s] += cut[s]
+    return [torch.cat(o) for o in outs]
+
+
+CUTS = [(5, 1), (1, 1), (2, 0), (1, 3), (17, 1), (1, 16), (0, 2), (33, 1), (1, 1), (2, 40)]      # 63 and 66 rows
+
+
+def mixer_case(kind, dtype, seed=0):
+    """(part, plain function over one sequence) of one mixer kind at sizes of its own."""
+    from leone_amd.parts import MIXERS, POSITIONS, PartSpec
+    gen = torch.Generator().manual_seed(seed)
+    width, eps = 48, 1e-5
+
+    def mat(rows, cols, scale=1.5):
+        return (torch.randn(rows, cols, generator=gen) * scale / math.sqrt(cols)).to(dtype)
+
+    def vec(n, mean=0.0, spread=1.0):
+        return (mean + spread * torch.randn(n, generator=gen)).to(dtype)
+
+    if kind == "mlstm":
+        m = {"heads": 3, "dim": 24, "vdim": 40, "gate_cap": 7.0}
+        w = {"q": mat(72, width), "k": mat(72, width), "v": mat(120, width), "g": mat(120, width), "o": mat(width, 120),
+             "norm": vec(120, 1.0, 0.2), "i": mat(3, width, 4.0), "i.b": vec(3), "f": mat(3, width, 4.0), "f.b": vec(3, 1.0)}
+        spec = PartSpec("mlstm", dict(hidden=width, eps=eps, **m, q="q", k="k", v="v", g="g", o="o", norm="norm", i="i",
+                                      i_bias="i.b", f="f", f_bias="f.b"))
+        part = MIXERS.build(spec)
+        reference = lambda h, ww: plain.mlstm(h, ww, "", m, eps)
+    elif kind == "retention":
+        m = {"heads": 2, "dim": 40, "vdim": 72, "decay": [0.9, 0.999], "rot": {"dims": 16, "base": 300.0}}
+        w = {"q": mat(80, width), "k": mat(80, width), "v": mat(144, width), "g": mat(144, width), "o": mat(width, 144)}
+        rope = POSITIONS.build(PartSpec("rope_half_split", {"rotary_dim": 16, "theta": 300.0}))
+        rope.prepare(256, DEV)
+        spec = PartSpec("retention", dict(hidden=width, eps=eps, heads=2, dim=40, vdim=72, decay=m["decay"], position="rope",
+                                          q="q", k="k", v="v", g="g", o="o"))
+        part = MIXERS.build(spec, positions={"rope": rope})
+        reference = lambda h, ww: plain.retention(h, ww, "", m, list(range(h.shape[0])), eps)
+    elif kind == "channel_delta":
+        m = {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 16, "conv": 3}
+        w = {"q": mat(48, width), "k": mat(48, width), "v": mat(64, width), "q.conv": mat(48, 3, 1.0), "k.conv": mat(48, 3, 1.0),
+             "v.conv": mat(64, 3, 1.0), "b": mat(4, width, 3.0), "A_log": vec(4, -1.0, 0.5), "dt_bias": vec(96),
+             "a1": mat(12, width), "a2": mat(96, 12, 3.0), "g1": mat(8, width), "g2": mat(64, 8), "norm": vec(16, 1.0, 0.2),
+             "o": mat(width, 64)}
+        spec = PartSpec("channel_delta", dict(hidden=width, eps=eps, heads=4, kv_heads=2, dim=24, vdim=16, taps=3, a_rank=12,
+                                              g_rank=8, q="q", k="k", v="v", q_conv="q.conv", k_conv="k.conv", v_conv="v.conv",
+                                              b="b", A_log="A_log", dt_bias="dt_bias", a1="a1", a2="a2", g1="g1", g2="g2",
+                                              norm="norm", o="o"))
+        part = MIXERS.build(spec)
+        reference = lambda h, ww: plain.channel_delta(h, ww, "", m, eps)
+    else:
+        m = {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 40, "scale": 0.3, "rot": {"dims": 8, "base": 1000.0}}
+        w = {"q": mat(96, width, 4.0), "k": mat(48, width, 4.0), "v": mat(80, width), "g": mat(4, width, 3.0), "o": mat(width, 160)}
+        rope = POSITIONS.build(PartSpec("rope_half_split", {"rotary_dim": 8, "theta": 1000.0}))
+        rope.prepare(256, DEV)
+        spec = PartSpec("gqa_attention", dict(hidden=width, q_heads=4, kv_heads=2, head_dim=24, value_dim=40, qk_norm_eps=None,
+                                              window=None, scale=0.3, position="rope", float_output=True, q="q", k="k", v="v",
+                                              o="o", gate="g"))
+        part = MIXERS.build(spec, positions={"rope": rope})
+        reference = lambda h, ww: plain.softmax_attention(h, ww, "", m, list(range(h.shape[0])))
+    part.bind({k: v.to(DEV) for k, v in w.items()})
+    return part, reference, {k: v.to(plain.F) for k, v in w.items()}, width
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+@pytest.mark.parametrize("kind", ["mlstm", "retention", "channel_delta", "softmax"])
+def test_each_mixer_alone_in_cuts_of_every_size(kind, dtype_name):
+    """One mixer, two sequences in one batch, cut into steps of 1 to 40 rows, one sequence now and then left out:
+    against the plain function over each whole sequence.  State slots and pages start out as NaN."""
+    dtype = DTYPES[dtype_name]
+    part, reference, w, width = mixer_case(kind, dtype)
+    gen = torch.Generator().manual_seed(4)
+    hs = [torch.randn(sum(c[s] for c in CUTS), width, generator=gen).to(dtype) for s in (0, 1)]
+    got = run_mixer_in_cuts(part, hs, CUTS, dtype)
+    for s in (0, 1):
+        want = reference(hs[s].to(plain.F), w)
+        err = pu.relative_error(got[s].numpy(), want.numpy())
+        tol = 2e-5 if dtype_name == "float32" else 3e-2
+        assert np.isfinite(got[s].numpy()).all() and err.max() <= tol, (kind, s, int(err.argmax()), float(err.max()))
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_attention_finds_a_far_key_and_keys_at_page_borders(dtype_name):
+    """Keys that answer one query each are planted far back and on both sides of page borders (pages of 16); the
+    queries come in a prompt's portion and as single decoded tokens.  A key that is skipped, or one from another
+    place, changes the result by the size of a value, far above rounding."""
+    from leone_amd.parts import MIXERS, PartSpec
+    dtype = DTYPES[dtype_name]
+    width, dim, vdim, heads = 32, 16, 24, 2
+    eye = torch.zeros(heads * dim, width)
+    for h in range(heads):
+        eye[h * dim:(h + 1) * dim, :dim] = torch.eye(dim)
+    gen = torch.Generator().manual_seed(7)
+    w = {"q": eye.clone(), "k": eye.clone(), "v": torch.randn(heads * vdim, width, generator=gen) / 4,
+         "g": torch.zeros(heads, width), "o": torch.randn(width, heads * vdim, generator=gen) / 6}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    part = MIXERS.build(PartSpec("gqa_attention", dict(hidden=width, q_heads=heads, kv_heads=heads, head_dim=dim, value_dim=vdim,
+                                                       qk_norm_eps=None, window=None, scale=1.0, position=None, float_output=True,
+                                                       q="q", k="k", v="v", o="o", gate="g")))
+    part.bind({k: v.to(DEV) for k, v in w.items()})
+    steps_total = 300
+    h = torch.randn(steps_total, width, generator=gen) * 0.05
+    planted = {3: 280, 15: 281, 16: 282, 17: 283, 127: 284, 128: 285, 0: 290, 31: 291, 32: 292, 255: 295}     # key -> query
+    for n, (key_at, query_at) in enumerate(planted.items()):
+        direction = torch.zeros(width)
+        direction[n % dim] = 6.0
+        direction[(n * 5 + 3) % dim] += 6.0 if n >= dim else 0.0
+        h[key_at, :dim] = direction[:dim]
+        h[query_at, :dim] = direction[:dim]
+        h[key_at, dim:] = torch.randn(width - dim, generator=gen)      # what the value is made from
+    h = h.to(dtype)
+    m = {"heads": heads, "kv_heads": heads, "dim": dim, "vdim": vdim, "scale": 1.0, "rot": {"dims": 2, "base": 1.0}}
+    wp = {k: v.to(plain.F) for k, v in w.items()}
+    # the plain function always rotates: a base of 1 turns every position by the same angle per step on 2 dims only;
+    # those two dims are kept out of the test by zero weights
+    for name in ("q", "k"):
+        wp[name] = wp[name].clone()
+        for hd in range(heads):
+            wp[name][hd * dim] = 0
+            wp[name][hd * dim + 1] = 0
+    part_w = {k: v.to(dtype).to(DEV) for k, v in ((n, wp[n].float()) for n in wp)}
+    part.bind(dict(part_w))
+    want = plain.softmax_attention(h.to(plain.F), wp, "", m, list(range(steps_total)))
+    cuts = [(270, 1), (10, 1)] + [(1, 1)] * 20
+    hs = [h, h[:22]]
+    got = run_mixer_in_cuts(part, hs, [(a, b) for a, b in cuts], dtype)[0]
+    err = pu.relative_error(got.numpy(), want.numpy())
+    tol = 2e-5 if dtype_name == "float32" else 3e-2
+    assert err.max() <= tol, (int(err.argmax()), float(err.max()))
+    # the planted keys matter: without them the queries' rows come out differently by far more than the tolerance
+    bare = h.clone().to(plain.F)
+    for key_at in planted:
+        bare[key_at, :dim] = 0
+    moved = pu.relative_error(plain.softmax_attention(bare, wp, "", m, list(range(steps_total))).numpy(), want.numpy())
+    assert all(moved[q] > 20 * tol for q in planted.values())
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+@pytest.mark.parametrize("taps", [2, 4, 7])
+def test_input_convolution_across_steps(taps, dtype_name):
+    """The convolution's reach against portions shorter than it: one, two and three rows at a time, two requests."""
+    from leone_amd.parts import CONVS, PartSpec
+    dtype = DTYPES[dtype_name]
+    channels = 40
+    gen = torch.Generator().manual_seed(taps)
+    weight = (torch.randn(channels, taps, generator=gen) * 0.5).to(dtype)
+    part = CONVS.build(PartSpec("causal_conv", {"channels": channels, "taps": taps, "weights": ["w"], "add_input": True}))
+    part.bind({"w": weight.to(DEV)})
+    cuts = [(1, 2), (2, 1), (1, 0), (3, 1), (1, 1), (0, 5), (9, 1), (1, 1)]
+    hs = [torch.randn(sum(c[s] for c in cuts), channels, generator=gen) for s in (0, 1)]
+    state = torch.full((3, taps - 1, channels), float("nan"), device=DEV)
+    from leone_amd.parts.context import StateCacheView
+    at, outs = [0, 0], [[], []]
+    for cut in cuts:
+        present = [s for s in (0, 1) if cut[s]]
+        meta = [(e, at[s] + i) for e, s in enumerate(present) for i in range(cut[s])]
+        x = torch.cat([hs[s][at[s]:at[s] + cut[s]] for s in present]).to(DEV)
+        out = part.forward(x, step_of(meta, dtype, [(1, 2)[s] for s in present]), StateCacheView(True, state), dtype)
+        first = 0
+        for s in present:
+            outs[s].append(out[first:first + cut[s]].float().cpu())
+            first += cut[s]
+            at[s] += cut[s]
+    for s in (0, 1):
+        want = plain.input_convolution(hs[s].to(plain.F), weight.to(plain.F))
+        err = (torch.cat(outs[s]).double() - want).abs().max()
+        assert err <= (1e-5 if dtype_name == "float32" else 5e-2), (s, float(err))
+
+
+def test_layer_norm_with_the_norm_behind_a_sublayer_folded_in():
+    from leone_amd import ops
+    from leone_amd.parts import NORMS, PartSpec
+    gen = torch.Generator().manual_seed(3)
+    size = 100
+    norms = {}
+    for name in ("a", "b"):
+        norms[name] = NORMS.build(PartSpec("layernorm", {"size": size, "eps": 1e-5, "weight": name, "bias": name + ".b"}))
+        norms[name].tensors = {name: 1 + 0.3 * torch.randn(size, generator=gen), name + ".b": 0.2 * torch.randn(size, generator=gen)}
+        norms[name].bind({k: v.to(DEV) for k, v in norms[name].tensors.items()})
+    x = torch.randn(7, size, generator=gen) * 3 + 1
+    delta = torch.randn(7, size, generator=gen) * 5 - 2
+    ta, tb = norms["a"].tensors, norms["b"].tensors
+    summed = x.double() + plain.layer_norm(delta.double(), ta["a"].double(), ta["a.b"].double(), 1e-5)
+    want = plain.layer_norm(summed, tb["b"].double(), tb["b.b"].double(), 1e-5)
+    stream = x.to(DEV)
+    y = norms["b"].add_norm(stream, ops.NormedDelta(delta.to(DEV), norms["a"]), torch.float32)
+    assert (y.cpu().double() - want).abs().max() < 1e-5 and (stream.cpu().double() - summed).abs().max() < 1e-5
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    stream = x.to(DEV)
+    picked = norms["b"].add_norm(stream, ops.NormedDelta(delta.to(DEV), norms["a"]), torch.float32, rows=rows)
+    assert (picked.cpu().double() - want[[5, 0, 5]]).abs().max() < 1e-5 and torch.equal(stream.cpu(), x)
