@@ -343,8 +343,98 @@ def run_scenario(name: str, dtype: str = "bfloat16", layers: Optional[int] = Non
             "preemptions": sched.preemptions, "max_step_rows": sched.max_step_rows, "max_live": sched.max_live}
 
 
+# ---- another design beside its closest relative, layer for layer ------------------------------------------------
+# Pamevik at sizes that resemble a real model's layers (the cell sizes of published mLSTM, retention and delta-rule
+# models: eight heads of 128 to 256 key channels with values twice as wide, 16 delta heads of 128 x 128, attention
+# with four query heads a key head), and Qwen3 with the same width, layers and vocabulary beside it.
+DESIGN_SIZES = {
+    "w2048": dict(width=2048, layers=8, vocab=32768, batch=8, context=2048, prompt=2048),
+    "w4096": dict(width=4096, layers=8, vocab=32768, batch=8, context=2048, prompt=2048),
+}
+
+
+def pamevik_shape(width: int, layers: int, vocab: int, context: int) -> dict:
+    heads = width // 512
+    cell = {"type": "mlstm", "mixer": {"heads": heads, "dim": 256, "vdim": 512, "gate_cap": 15.0}, "mlp": None}
+    pair = {"type": "parallel", "mlp": {"kind": "dense", "ff": 3 * width},
+            "mixer": {"left": {"heads": width // 128, "kv_heads": width // 512, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                               "rot": {"dims": 128, "base": 1000000.0}},
+                      "right": {"heads": heads, "dim": 128, "vdim": 256, "rot": {"dims": 64, "base": 10000.0},
+                                "decay": [1.0 - 2.0 ** (-5 - h) for h in range(heads)]}}}
+    rule = {"type": "channel_delta", "mlp": None,
+            "mixer": {"heads": width // 128, "kv_heads": width // 256, "dim": 128, "vdim": 128, "conv": 4, "a_rank": 64, "g_rank": 64}}
+    order = [cell, cell, pair, rule]
+    return {"architecture": "Pamevik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "canon": {"taps": 4},
+            "max_positions": max(4096, context + 64), "layers": [order[i % 4] for i in range(layers)]}
+
+
+def state_bytes_per_request(model) -> int:
+    """Bytes of per-request state a decode step reads and writes back (both ways counted)."""
+    total = 0
+    for need in model.cache_needs().values():
+        if not getattr(need, "paged", False):
+            count = 1
+            for extent in need.shape:
+                count *= extent
+            total += 2 * count * 4
+    return total
+
+
+def run_design(name: str, sizes: List[str], steps: int, warmup: int) -> dict:
+    """Decode and prefill throughput of ``name`` ("pamevik") at DESIGN_SIZES, each beside Qwen3 at the same width,
+    layers and vocabulary, with a per-operation table of a decode step and of the prompt's step for both."""
+    import torch
+    from .architectures import config_from_dict
+    from .engine.engine import Engine, StepEntry
+    from .ops.profile import Recorder
+    from .runtime import random_model
+
+    def measure(raw: dict, size: dict) -> dict:
+        model = random_model(config_from_dict(raw), seed=0, dtype="bfloat16")
+        batch, context, prompt = size["batch"], size["context"], size["prompt"]
+        pages = batch * (context // 64 + 2) + prompt // 64 + 1
+        engine = Engine(model, num_pages=pages, page_tokens=64, max_requests=batch + 1, max_context=max(context, prompt) + 64)
+        start = context - steps - warmup - 5
+        elapsed, mean_context, profiled = time_decode(engine, batch, start, steps, warmup, profile_steps=4)
+        step_bytes = decode_bytes(model, batch, mean_context) + batch * state_bytes_per_request(model)
+        out = {"decode_tok_s": round(batch * steps / elapsed, 1), "decode_ms_per_step": round(elapsed / steps * 1e3, 3),
+               "decode_gb_per_step": round(step_bytes / 1e9, 3), "decode_gbs": round(step_bytes / (elapsed / steps) / 1e9, 1),
+               "decode_operations_us": {k: v["us"] for k, v in kernel_table(profiled, model, batch, mean_context).items()}}
+        seconds = time_prefill(engine, prompt)
+        out.update(prefill_tok_s=round(prompt / seconds, 1), prefill_ms=round(seconds * 1e3, 3))
+        recorder = Recorder(1)
+        tokens = [(i * 7919) % engine.vocab_size for i in range(prompt)]
+        recorder.begin_step()
+        engine.step([StepEntry("profiled prompt", tokens, [prompt - 1])])
+        recorder.end_step(prompt)
+        engine.release("profiled prompt")
+        out["prefill_operations_us"] = {k: round(v * 1e6, 1) for k, v in recorder.profile.seconds_by_operation.items()}
+        del engine, model
+        torch.cuda.empty_cache()
+        return out
+
+    points = {}
+    for key in sizes:
+        size = DESIGN_SIZES[key]
+        new = measure(pamevik_shape(size["width"], size["layers"], size["vocab"], max(size["context"], size["prompt"])), size)
+        beside = measure(dict(QWEN3_8B, num_hidden_layers=size["layers"], hidden_size=size["width"],
+                              num_attention_heads=size["width"] // 128, num_key_value_heads=size["width"] // 512,
+                              intermediate_size=3 * size["width"], vocab_size=size["vocab"],
+                              max_position_embeddings=max(4096, size["context"] + 64)), size)
+        points[key] = {"sizes": size, name: new, "qwen3": beside}
+    first = points[sizes[0]]
+    return {"metric": f"decode tok/s ({name} beside qwen3 at equal width, layers and vocabulary)",
+            "value": first[name]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": first[name]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic", "config": {"model": name, "sizes": sizes}, "points": points}
+
+
 def main(argv: Optional[List[str]] = None) -> int:
     parser = argparse.ArgumentParser(prog="bench.py")
+    parser.add_argument("--design", choices=["pamevik"],
+                        help="instead of the headline figure: this design at a few layer sizes beside Qwen3 at equal size "
+                             "(decode and prefill throughput, per-operation times)")
+    parser.add_argument("--design-sizes", default="w2048,w4096", help="which of " + ", ".join(sorted(DESIGN_SIZES)))
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=64)
     parser.add_argument("--warmup", type=int, default=8)
@@ -376,6 +466,9 @@ def main(argv: Optional[List[str]] = None) -> int:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
 
+    if args.design:
+        print(json.dumps(run_design(args.design, args.design_sizes.split(","), args.steps, args.warmup)), flush=True)
+        return 0
     if args.scenario:
         print(json.dumps(run_scenario(args.scenario, args.dtype, args.layers, args.tuned_products)), flush=True)
         return 0

@@ -2,7 +2,7 @@
 //
 //   add_layernorm     x += LayerNorm_a(delta) (if a delta comes), y = LayerNorm_b(x): the norm after one
 //                     sublayer, the residual sum and the norm before the next in one pass over the row
-//   entry_spans       first and last row of every entry of a step, from the row -> entry map
+//   entry_spans       first row and end of every entry of a step, and its state slot, from the row -> entry map
 //   causal_conv       out[t] = (in[t] if asked) + sum_j w[c, j] * in[t - (taps - 1) + j], per channel, the
 //                     rows before a portion taken from the request's state (its last taps - 1 inputs)
 //   causal_conv_state leaves the last taps - 1 inputs of every entry behind as the new state
@@ -68,12 +68,17 @@ add_layernorm_kernel(float* __restrict__ x, const float* __restrict__ delta, Any
         yr[i] = from_float<TOut>((row_buf[i] - mean) * rstd * load_any(w, i) + load_any(b, i));
 }
 
-__global__ void entry_spans_kernel(const int* __restrict__ row_entry, int rows, int* __restrict__ spans) {
+__global__ void entry_spans_kernel(const int* __restrict__ row_entry, const int* __restrict__ positions,
+                                   const int* __restrict__ entry_slots, int rows, int* __restrict__ spans) {
     const int r = blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= rows) return;
     const int e = row_entry[r];
-    if (r == 0 || row_entry[r - 1] != e) spans[2 * e] = r;
-    if (r == rows - 1 || row_entry[r + 1] != e) spans[2 * e + 1] = r + 1;
+    if (r == 0 || row_entry[r - 1] != e) {
+        spans[4 * e] = r;
+        spans[4 * e + 2] = positions[r] == 0 ? -1 : entry_slots[e];     // a sequence's start: from zeros
+        spans[4 * e + 3] = entry_slots[e];
+    }
+    if (r == rows - 1 || row_entry[r + 1] != e) spans[4 * e + 1] = r + 1;
 }
 
 enum Activation : int { kActNone = 0, kActSigmoid = 1, kActSilu = 2 };
@@ -116,7 +121,7 @@ __global__ void causal_conv_state_kernel(const TIn* __restrict__ in, long in_str
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     const int e = blockIdx.y;
     if (c >= channels) return;
-    const int first = spans[2 * e], n = spans[2 * e + 1] - first;
+    const int first = spans[4 * e], n = spans[4 * e + 1] - first;
     const int start = positions[first];
     float* mine = state + (static_cast<long>(entry_slots[e]) * (taps - 1)) * channels + c;
     float keep[kMaxTaps - 1];
@@ -227,9 +232,10 @@ extern "C" int leone_add_layernorm(float* x, const float* delta, const void* dw,
     return 0;
 }
 
-extern "C" int leone_entry_spans(const int* row_entry, int rows, int* spans, hipStream_t stream) {
-    LEONE_REQUIRE(row_entry && spans && rows > 0, "entry_spans: needs a row map");
-    entry_spans_kernel<<<ceil_div(rows, 256), 256, 0, stream>>>(row_entry, rows, spans);
+extern "C" int leone_entry_spans(const int* row_entry, const int* positions, const int* entry_slots, int rows, int* spans,
+                                 hipStream_t stream) {
+    LEONE_REQUIRE(row_entry && positions && entry_slots && spans && rows > 0, "entry_spans: needs a row map");
+    entry_spans_kernel<<<ceil_div(rows, 256), 256, 0, stream>>>(row_entry, positions, entry_slots, rows, spans);
     LEONE_LAUNCH_CHECK("entry_spans");
     return 0;
 }

@@ -206,8 +206,10 @@ int leone_sample_truncated(const float* logits, const double* params, int* out, 
 int leone_add_layernorm(float* x, const float* delta, const void* dw, const void* db, float deps, const void* w,
                         const void* b, int w_dtype, float eps, void* y, int y_dtype, const int* rows, int n_out,
                         int hidden, hipStream_t stream);
-// spans[2e], spans[2e + 1]: first row and end of entry e (an entry's rows are consecutive).
-int leone_entry_spans(const int* row_entry, int rows, int* spans, hipStream_t stream);
+// spans[4e .. 4e + 3]: first row and end of entry e (an entry's rows are consecutive), the state slot it reads
+// (-1 at a sequence's start: zeros) and the one it writes.
+int leone_entry_spans(const int* row_entry, const int* positions, const int* entry_slots, int rows, int* spans,
+                      hipStream_t stream);
 // A causal convolution over time per channel, w [channels, taps] with the last tap on the current row; the
 // rows before a portion come from state [slots, taps - 1, channels] (float), which is brought up to date if asked.
 // act: 0 none, 1 sigmoid, 2 silu.
@@ -227,16 +229,24 @@ int leone_head_gate(void* out, int dtype, const float* gate, long gate_stride, i
                     hipStream_t stream);
 // The matrix-memory recurrences (see recurrent.hip); key sizes up to leone_scan_max_dim().
 int leone_scan_max_dim();
-int leone_outer_scan(const float* proj, long stride, int q_off, int k_off, int v_off, int i_off, int f_off,
-                     const void* i_bias, const void* f_bias, int bias_dtype, float cap, const float* decay,
-                     float q_scale, float k_scale, const float* cos_table, const float* sin_table, int rotary_dim,
-                     int table_positions, float* state, long slot_stride, int write_state, const int* spans,
-                     const int* entry_slots, const int* positions, int entries, float* out, float* dot, float* top,
+// segments: n x (first row, end, index of the state read or -1 for zeros, index of the state written or -1).
+int leone_exp_gates(const float* proj, long stride, int i_off, int f_off, const void* i_bias, const void* f_bias,
+                    int bias_dtype, float cap, const int* spans, int entries, float* state, long slot_stride,
+                    long head_stride, long top_at, int write_state, float* coef, float* top, int heads, hipStream_t stream);
+int leone_outer_scan(const float* proj, long stride, int q_off, int k_off, int v_off, const float* coef,
+                     const float* decay, int no_input, int accumulate, int norm_column, float q_scale, float k_scale,
+                     const float* cos_table, const float* sin_table, int rotary_dim, int table_positions,
+                     const int* positions, const int* segments, int n_segments, const float* state_in, long in_stride,
+                     float* state_out, long out_stride, long head_stride, float* decay_product, float* out, float* dot,
                      int heads, int dim, int vdim, hipStream_t stream);
+int leone_outer_chain(const int* links, int n_links, float* work, long work_stride, const float* product, float* state,
+                      long slot_stride, long head_stride, int per_head, int heads, int write_state, hipStream_t stream);
 int leone_delta_scan(const float* qkv, long stride, int q_off, int k_off, int v_off, const float* beta,
                      long beta_stride, const float* step, long step_stride, const void* rate_log,
-                     const void* step_bias, int vec_dtype, float q_scale, float unit_eps, float* state,
-                     long slot_stride, int write_state, const int* spans, const int* entry_slots,
-                     const int* positions, int entries, float* out, int heads, int kv_heads, int dim, int vdim,
+                     const void* step_bias, int vec_dtype, float q_scale, float unit_eps, int no_input, int accumulate,
+                     const int* segments, int n_segments, const float* state_in, long in_stride, float* state_out,
+                     long out_stride, float* transition, float* out, int heads, int kv_heads, int dim, int vdim,
                      hipStream_t stream);
+int leone_delta_chain(const int* links, int n_links, float* work, long work_stride, const float* transition, float* state,
+                      long slot_stride, int heads, int dim, int vdim, int write_state, hipStream_t stream);
 }

@@ -1114,16 +1114,56 @@ def add_layernorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional
 
 
 def entry_spans(step) -> torch.Tensor:
-    """int32 ``[entries, 2]`` on the device: first row and end of every entry's rows in the step, made once a
-    step from the row -> entry map (so that it is there too when a step is replayed from a recording)."""
+    """int32 ``[entries, 4]`` on the device: first row and end of every entry's rows in the step, the state slot
+    it reads (-1 at a sequence's start: it starts from zeros) and the slot it writes; made once a step from
+    the row -> entry map (so that it is there too when a step is replayed from a recording)."""
     spans = getattr(step, "spans", None)
     if spans is None:
         entries = step.entry_slots.numel()
-        spans = torch.empty((entries, 2), dtype=torch.int32, device=step.row_entry.device)
-        call("leone_entry_spans", _dev(step.row_entry, "row map", torch.int32, (step.rows,)), step.rows,
-             _dev(spans, "spans"), _stream())
+        spans = torch.empty((entries, 4), dtype=torch.int32, device=step.row_entry.device)
+        call("leone_entry_spans", _dev(step.row_entry, "row map", torch.int32, (step.rows,)),
+             _dev(step.positions, "positions", torch.int32, (step.rows,)), _dev(step.entry_slots, "slots", torch.int32),
+             step.rows, _dev(spans, "spans"), _stream())
         step.spans = spans
     return spans
+
+
+# Rows of a chunk when a long portion's recurrence is walked chunk by chunk, side by side, and the portions that
+# are (at least so many rows): (chunk, from).  The outer-product recurrences chain their chunks by a factor, the
+# delta rule by a matrix product a chunk, so its chunks are longer.
+OUTER_CHUNKS = (64, 256)
+DELTA_CHUNKS = (256, 512)
+
+
+def chunk_plan(step, chunk: int, chunked_from: int):
+    """How the recurrences of a step with long portions are walked (``outer_scan``): None if the step has none (or
+    is replayed from a recording: then the host does not know its entries).  Else int32 tables on the device:
+    ``chunks`` ``[c, 4]`` (first row, end, -1, chunk index) of the long portions' chunks, ``again`` the same chunks
+    reading (chunk index, -1), ``links`` ``[l, 4]`` (state slot, whether the sequence starts here, first chunk, end)
+    one a long portion, and ``short`` ``[s, 4]`` the other entries as single segments from and into their slots."""
+    plans = step.plan if isinstance(step.plan, dict) else {}
+    step.plan = plans
+    key = (chunk, chunked_from)
+    if key in plans:
+        return plans[key]
+    plans[key] = None
+    if not any(e.count >= chunked_from for e in step.entries):
+        return None
+    chunks, again, links, short = [], [], [], []
+    for e in step.entries:
+        if e.count >= chunked_from:
+            first_chunk = len(chunks)
+            for at in range(0, e.count, chunk):
+                rows = (e.first_row + at, e.first_row + min(at + chunk, e.count))
+                again.append(rows + (len(chunks), -1))
+                chunks.append(rows + (-1, len(chunks)))
+            links.append((e.slot, 1 if e.start == 0 else 0, first_chunk, len(chunks)))
+        else:
+            short.append((e.first_row, e.first_row + e.count, -1 if e.start == 0 else e.slot, e.slot))
+    flat = torch.tensor(chunks + again + links + short, dtype=torch.int32).to(step.device)
+    c, l = len(chunks), len(links)
+    plans[key] = {"chunks": flat[:c], "again": flat[c:2 * c], "links": flat[2 * c:2 * c + l], "short": flat[2 * c + l:]}
+    return plans[key]
 
 
 def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, step, out_dtype: torch.dtype,
@@ -1220,31 +1260,57 @@ def outer_scan(proj: torch.Tensor, columns: dict, state: torch.Tensor, step, hea
     first column of q, k and v (and, with ``gates``, of the input and forget gates' pre-activations "i", "f").
     ``gates`` = {"i_bias", "f_bias", "cap"}: exponential gates with a running maximum that starts at 0; else
     ``decay`` (float32 ``[heads]``) with b = 1.  ``cos``/``sin``: rotary tables for q and k.
-    Returns o float32 ``[rows, heads * vdim]`` and, with gates, (dot, top) for ``head_norm_gate``."""
+    Returns o float32 ``[rows, heads * vdim]`` and, with gates, (dot, top) for ``head_norm_gate``.
+
+    Single tokens and short portions are walked row by row.  A long portion (``OUTER_CHUNKS``) is cut into chunks
+    that are walked side by side: every chunk from zeros, the chunks' end states chained, every chunk once more
+    from the state it starts with."""
     rows, width = proj.shape
     per_head = dim * vdim + (dim + 1 if gates else 0)
-    if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (heads, per_head):
+    if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (heads, per_head) or not state.is_contiguous():
         raise KernelError(f"outer_scan: state {tuple(state.shape)} is not [slots, {heads}, {per_head}] float32")
     spans = entry_spans(step)
-    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=proj.device)
-    dot = top = None
+    device = proj.device
+    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=device)
+    dot = top = coef = None
     if gates:
-        dot = torch.empty((rows, heads), dtype=torch.float32, device=proj.device)
-        top = torch.empty((rows, heads), dtype=torch.float32, device=proj.device)
+        dot = torch.empty((rows, heads), dtype=torch.float32, device=device)
+        top = torch.empty((rows, heads), dtype=torch.float32, device=device)
+        coef = torch.empty((rows, heads, 2), dtype=torch.float32, device=device)
         if gates["i_bias"].dtype != gates["f_bias"].dtype:
             raise KernelError("outer_scan: the gates' biases must share one type")
+        call("leone_exp_gates", _dev(proj, "projection", torch.float32), width, columns["i"], columns["f"],
+             _dev(gates["i_bias"], "i bias", None, (heads,)), _dev(gates["f_bias"], "f bias", None, (heads,)),
+             _code(gates["i_bias"], "i bias"), float(gates["cap"]), _dev(spans, "spans"), spans.shape[0],
+             _dev(state, "state"), state.stride(0), per_head, dim * vdim + dim, 1 if write_state else 0,
+             _dev(coef, "coefficients"), _dev(top, "top"), heads, _stream())
     rotary_dim = 2 * cos.shape[1] if cos is not None else 0
-    call("leone_outer_scan", _dev(proj, "projection", torch.float32), width, columns["q"], columns["k"], columns["v"],
-         columns["i"] if gates else -1, columns["f"] if gates else -1,
-         _dev(gates["i_bias"], "i bias", None, (heads,)) if gates else 0,
-         _dev(gates["f_bias"], "f bias", None, (heads,)) if gates else 0,
-         _code(gates["i_bias"], "i bias") if gates else F32, float(gates["cap"]) if gates else 0.0,
-         _dev(decay, "decay", torch.float32, (heads,)) if decay is not None else 0, float(q_scale), float(k_scale),
-         _dev(cos, "rope cos", torch.float32), _dev(sin, "rope sin", torch.float32), rotary_dim,
-         cos.shape[0] if cos is not None else 0, _dev(state, "state"), state.stride(0), 1 if write_state else 0,
-         _dev(spans, "spans"), _dev(step.entry_slots, "slots", torch.int32),
-         _dev(step.positions, "positions", torch.int32, (rows,)), spans.shape[0], _dev(out, "out"),
-         _dev(dot, "dot"), _dev(top, "top"), heads, dim, vdim, _stream())
+
+    def walk(segments, state_in, state_out, no_input=False, accumulate=False, product=None):
+        call("leone_outer_scan", _dev(proj, "projection", torch.float32), width, columns["q"], columns["k"], columns["v"],
+             _dev(coef, "coefficients"), _dev(decay, "decay", torch.float32, (heads,)) if decay is not None else 0,
+             1 if no_input else 0, 1 if accumulate else 0, 1 if gates else 0, float(q_scale), float(k_scale),
+             _dev(cos, "rope cos", torch.float32), _dev(sin, "rope sin", torch.float32), rotary_dim,
+             cos.shape[0] if cos is not None else 0, _dev(step.positions, "positions", torch.int32, (rows,)),
+             _dev(segments, "segments", torch.int32), segments.shape[0],
+             _dev(state_in, "state read"), state_in.stride(0) if state_in is not None else 0,
+             _dev(state_out, "state written"), state_out.stride(0) if state_out is not None else 0, per_head,
+             _dev(product, "decay products"), _dev(out, "out"), _dev(dot, "dot"), heads, dim, vdim, _stream())
+
+    plan = chunk_plan(step, *OUTER_CHUNKS)
+    if plan is None:
+        walk(spans, state, state if write_state else None)
+    else:
+        chunks = plan["chunks"]
+        work = torch.empty((chunks.shape[0], heads, per_head), dtype=torch.float32, device=device)
+        product = torch.empty((chunks.shape[0], heads), dtype=torch.float32, device=device)
+        walk(chunks, None, work, product=product)
+        call("leone_outer_chain", _dev(plan["links"], "links", torch.int32), plan["links"].shape[0], _dev(work, "work"),
+             work.stride(0), _dev(product, "decay products"), _dev(state, "state"), state.stride(0), per_head,
+             dim * vdim + (dim if gates else 0), heads, 1 if write_state else 0, _stream())
+        walk(plan["again"], work, None, no_input=True, accumulate=True)
+        if plan["short"].shape[0]:
+            walk(plan["short"], state, state if write_state else None)
     return (out, (dot, top)) if gates else (out, None)
 
 
@@ -1256,20 +1322,43 @@ def delta_scan(qkv: torch.Tensor, columns: dict, beta: torch.Tensor, step_size: 
     made unit vectors per head (x / sqrt(sum x^2 + unit_eps)) and q times ``q_scale``.  ``qkv`` float32 rows
     holding q and k (``kv_heads`` heads of ``dim``) and v (``heads`` of ``vdim``) at ``columns``; ``beta`` float32
     ``[rows, heads]`` and ``step_size`` ``[rows, heads * dim]`` may be slices of wider rows.  ``state`` float32
-    ``[slots, heads, dim, vdim]``.  Returns o float32 ``[rows, heads * vdim]``."""
+    ``[slots, heads, dim, vdim]``.  Returns o float32 ``[rows, heads * vdim]``.
+
+    Long portions are walked in chunks side by side, as in ``outer_scan``; what a chunk's rows do to a state that
+    comes in is no mere factor here but a matrix ``[dim, dim]``, which the first walk finds by carrying the unit
+    vectors along as further columns."""
     rows = qkv.shape[0]
-    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, dim, vdim):
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, dim, vdim) or not state.is_contiguous():
         raise KernelError(f"delta_scan: state {tuple(state.shape)} is not [slots, {heads}, {dim}, {vdim}] float32")
     if rate_log.dtype != step_bias.dtype:
         raise KernelError("delta_scan: rate and step bias must share one type")
     spans = entry_spans(step)
-    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=qkv.device)
+    device = qkv.device
+    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=device)
     beta_at, beta_stride = _strided_rows(beta, "delta_scan beta", rows, heads)
     step_at, step_stride = _strided_rows(step_size, "delta_scan step", rows, heads * dim)
-    call("leone_delta_scan", _dev(qkv, "q, k, v", torch.float32), qkv.shape[1], columns["q"], columns["k"], columns["v"],
-         beta_at, beta_stride, step_at, step_stride, _dev(rate_log, "rate", None, (heads,)),
-         _dev(step_bias, "step bias", None, (heads * dim,)), _code(rate_log, "rate"), float(q_scale), float(unit_eps),
-         _dev(state, "state"), state.stride(0), 1 if write_state else 0, _dev(spans, "spans"),
-         _dev(step.entry_slots, "slots", torch.int32), _dev(step.positions, "positions", torch.int32, (rows,)),
-         spans.shape[0], _dev(out, "out"), heads, kv_heads, dim, vdim, _stream())
+
+    def walk(segments, state_in, state_out, no_input=False, accumulate=False, transition=None):
+        call("leone_delta_scan", _dev(qkv, "q, k, v", torch.float32), qkv.shape[1], columns["q"], columns["k"], columns["v"],
+             beta_at, beta_stride, step_at, step_stride, _dev(rate_log, "rate", None, (heads,)),
+             _dev(step_bias, "step bias", None, (heads * dim,)), _code(rate_log, "rate"), float(q_scale), float(unit_eps),
+             1 if no_input else 0, 1 if accumulate else 0, _dev(segments, "segments", torch.int32), segments.shape[0],
+             _dev(state_in, "state read"), state_in.stride(0) if state_in is not None else 0,
+             _dev(state_out, "state written"), state_out.stride(0) if state_out is not None else 0,
+             _dev(transition, "transitions"), _dev(out, "out"), heads, kv_heads, dim, vdim, _stream())
+
+    plan = chunk_plan(step, *DELTA_CHUNKS)
+    if plan is None:
+        walk(spans, state, state if write_state else None)
+    else:
+        chunks = plan["chunks"]
+        work = torch.empty((chunks.shape[0], heads, dim, vdim), dtype=torch.float32, device=device)
+        transition = torch.empty((chunks.shape[0], heads, dim, dim), dtype=torch.float32, device=device)
+        walk(chunks, None, work, transition=transition)
+        call("leone_delta_chain", _dev(plan["links"], "links", torch.int32), plan["links"].shape[0], _dev(work, "work"),
+             work.stride(0), _dev(transition, "transitions"), _dev(state, "state"), state.stride(0), heads, dim, vdim,
+             1 if write_state else 0, _stream())
+        walk(plan["again"], work, None, no_input=True, accumulate=True)
+        if plan["short"].shape[0]:
+            walk(plan["short"], state, state if write_state else None)
     return out

@@ -53,17 +53,21 @@ _PROTOTYPES = {
     "leone_top_candidates": [P, P, P, P, c_int, c_int, c_int, P],
     "leone_sample_truncated": [P, P, P, c_int, c_int, P],
     "leone_add_layernorm": [P, P, P, P, c_float, P, P, c_int, c_float, P, c_int, P, c_int, c_int, P],
-    "leone_entry_spans": [P, c_int, P, P],
+    "leone_entry_spans": [P, P, P, c_int, P, P],
     "leone_causal_conv": [P, c_int, ctypes.c_long, P, c_int, ctypes.c_long, P, c_int, P, c_int, P, c_int, P, P, P, c_int,
                           c_int, c_int, c_int, c_int, P],
     "leone_head_norm_gate": [P, P, P, P, c_int, c_int, P, ctypes.c_long, c_int, c_float, P, c_int, c_int, c_int, c_int, P],
     "leone_rms_mix": [P, P, c_int, c_int, c_float, c_float, P, c_int, c_int, P],
     "leone_relu_squared": [P, P, c_int, ctypes.c_long, P],
     "leone_head_gate": [P, c_int, P, ctypes.c_long, c_int, c_int, c_int, P],
-    "leone_outer_scan": [P, ctypes.c_long, c_int, c_int, c_int, c_int, c_int, P, P, c_int, c_float, P, c_float, c_float,
-                         P, P, c_int, c_int, P, ctypes.c_long, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, P],
+    "leone_exp_gates": [P, ctypes.c_long, c_int, c_int, P, P, c_int, c_float, P, c_int, P, ctypes.c_long, ctypes.c_long,
+                        ctypes.c_long, c_int, P, P, c_int, P],
+    "leone_outer_scan": [P, ctypes.c_long, c_int, c_int, c_int, P, P, c_int, c_int, c_int, c_float, c_float, P, P, c_int, c_int,
+                         P, P, c_int, P, ctypes.c_long, P, ctypes.c_long, ctypes.c_long, P, P, P, c_int, c_int, c_int, P],
+    "leone_outer_chain": [P, c_int, P, ctypes.c_long, P, P, ctypes.c_long, ctypes.c_long, c_int, c_int, c_int, P],
     "leone_delta_scan": [P, ctypes.c_long, c_int, c_int, c_int, P, ctypes.c_long, P, ctypes.c_long, P, P, c_int, c_float,
-                         c_float, P, ctypes.c_long, c_int, P, P, P, c_int, P, c_int, c_int, c_int, c_int, P],
+                         c_float, c_int, c_int, P, c_int, P, ctypes.c_long, P, ctypes.c_long, P, P, c_int, c_int, c_int, c_int, P],
+    "leone_delta_chain": [P, c_int, P, ctypes.c_long, P, P, ctypes.c_long, c_int, c_int, c_int, c_int, P],
 }
 
 

@@ -35,6 +35,18 @@ OPERATIONS = {
     "leone_argmax": "argmax",
     "leone_sample_temperature": "sample",
     "leone_top_candidates": "sample",
+    "leone_add_layernorm": "layer norm",
+    "leone_entry_spans": "entry spans",
+    "leone_causal_conv": "causal conv",
+    "leone_head_norm_gate": "head norm gate",
+    "leone_rms_mix": "branch mix",
+    "leone_relu_squared": "relu squared",
+    "leone_head_gate": "head gate",
+    "leone_outer_scan": "outer scan",
+    "leone_outer_chain": "outer scan",
+    "leone_exp_gates": "exp gates",
+    "leone_delta_scan": "delta scan",
+    "leone_delta_chain": "delta scan",
 }
 LIBRARY_PRODUCT = "gemm library"
 ORDER = ["embed", "norm", "gemv fused", "gemm rows", LIBRARY_PRODUCT, "gemm f32", "qknorm rope kv", "attention", "swiglu",

@@ -50,6 +50,8 @@ class StepContext:
     tiled: Dict[object, TiledRows] = field(default_factory=dict)
     # int32 [entries, 2] on the device: first row and end of every entry (``ops.entry_spans`` makes it on first use).
     spans: Optional[torch.Tensor] = None
+    # How the recurrences of a step with long portions are walked (``ops.chunk_plan`` makes it on first use).
+    plan: object = None
 
 
 @dataclass
