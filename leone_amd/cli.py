@@ -232,8 +232,10 @@ def cmd_doctor(args) -> int:
         config = config_from_dir(args.model)
         print(f"architecture: {config.architecture}")
         print(f"context limit: {config.max_position_embeddings}")
-        model = DecoderModel(model_spec_for(config), torch.float32, "cpu")
         files = ModelFiles(args.model)
+        if hasattr(config, "with_shapes"):       # a design that leaves some sizes to the tensors' shapes
+            config = config.with_shapes({name: tuple(entry.shape) for name, entry in files.entries.items()})
+        model = DecoderModel(model_spec_for(config), torch.float32, "cpu")
         total = 0
         by_type = {}
         for entry in files.entries.values():

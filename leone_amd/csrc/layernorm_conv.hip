@@ -18,7 +18,7 @@
 
 namespace leone {
 
-constexpr int kNormThreads = 256;
+constexpr int kNormThreads = 1024;     // few elements a thread: a row is a handful of trips to memory, not one per element
 constexpr int kMaxTaps = 16;
 
 // Mean and inverse deviation of n values read through f(i); every thread gets both.
@@ -40,19 +40,32 @@ __device__ inline void mean_rstd(F value, int n, float eps, float* scratch, floa
 template <typename TOut>
 __global__ void __launch_bounds__(kNormThreads)
 add_layernorm_kernel(float* __restrict__ x, const float* __restrict__ delta, AnyVec dw, AnyVec db, float deps,
-                     AnyVec w, AnyVec b, float eps, TOut* __restrict__ y, const int* __restrict__ rows, int hidden) {
-    extern __shared__ float row_buf[];
+                     AnyVec w, AnyVec b, float eps, TOut* __restrict__ y, const int* __restrict__ rows, int hidden,
+                     AnyVec conv, int taps, float* __restrict__ conv_state, int write_state,
+                     const int* __restrict__ positions, const int* __restrict__ row_entry, const int* __restrict__ entry_slots,
+                     int stage_delta) {
+    extern __shared__ float row_buf[];          // the row; behind it, if there is room, the delta's row
     __shared__ float scratch[kNormThreads / kWave];
     const long src = rows ? rows[blockIdx.x] : blockIdx.x;
     float* xr = x + src * hidden;
     if (delta) {
         const float* dr = delta + src * hidden;
-        float mean = 0.f, rstd = 1.f;
-        if (dw.ptr) mean_rstd([&](int i) { return dr[i]; }, hidden, deps, scratch, mean, rstd);
+        // both rows are fetched once, side by side; the passes after that read shared memory
+        float* staged = stage_delta ? row_buf + hidden : nullptr;
         for (int i = threadIdx.x; i < hidden; i += kNormThreads) {
-            float d = dr[i];
+            row_buf[i] = xr[i];
+            if (staged) staged[i] = dr[i];
+        }
+        __syncthreads();
+        float mean = 0.f, rstd = 1.f;
+        if (dw.ptr) {
+            if (staged) mean_rstd([&](int i) { return staged[i]; }, hidden, deps, scratch, mean, rstd);
+            else mean_rstd([&](int i) { return dr[i]; }, hidden, deps, scratch, mean, rstd);
+        }
+        for (int i = threadIdx.x; i < hidden; i += kNormThreads) {
+            float d = staged ? staged[i] : dr[i];
             if (dw.ptr) d = (d - mean) * rstd * load_any(dw, i) + load_any(db, i);
-            const float t = xr[i] + d;
+            const float t = row_buf[i] + d;
             row_buf[i] = t;
             if (!rows) xr[i] = t;
         }
@@ -64,8 +77,27 @@ add_layernorm_kernel(float* __restrict__ x, const float* __restrict__ delta, Any
     float mean, rstd;
     mean_rstd([&](int i) { return row_buf[i]; }, hidden, eps, scratch, mean, rstd);
     TOut* yr = y + static_cast<long>(blockIdx.x) * hidden;
-    for (int i = threadIdx.x; i < hidden; i += kNormThreads)
-        yr[i] = from_float<TOut>((row_buf[i] - mean) * rstd * load_any(w, i) + load_any(b, i));
+    if (!conv.ptr) {
+        for (int i = threadIdx.x; i < hidden; i += kNormThreads)
+            yr[i] = from_float<TOut>((row_buf[i] - mean) * rstd * load_any(w, i) + load_any(b, i));
+        return;
+    }
+    // A step of single rows, every row another request: the input convolution of the sublayer that reads this
+    // norm is done here, h + conv(h) over the request's last inputs, and its state moved on by this row.
+    const int pos = positions[blockIdx.x];
+    float* keep = conv_state + static_cast<long>(entry_slots[row_entry[blockIdx.x]]) * (taps - 1) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += kNormThreads) {
+        const float h = (row_buf[i] - mean) * rstd * load_any(w, i) + load_any(b, i);
+        float acc = 0.f;
+        for (int j = 0; j + 1 < taps; ++j) {                 // oldest input first
+            const float old = pos - (taps - 1 - j) < 0 ? 0.f : keep[static_cast<long>(j) * hidden + i];
+            acc = fmaf(load_any(conv, static_cast<long>(i) * taps + j), old, acc);
+            if (write_state && j > 0) keep[static_cast<long>(j - 1) * hidden + i] = old;
+        }
+        acc = fmaf(load_any(conv, static_cast<long>(i) * taps + taps - 1), h, acc);
+        if (write_state) keep[static_cast<long>(taps - 2) * hidden + i] = h;
+        yr[i] = from_float<TOut>(h + acc);
+    }
 }
 
 __global__ void entry_spans_kernel(const int* __restrict__ row_entry, const int* __restrict__ positions,
@@ -93,7 +125,7 @@ template <typename TIn, typename TOut>
 __global__ void causal_conv_kernel(const TIn* __restrict__ in, long in_stride, TOut* __restrict__ out, long out_stride,
                                    AnyVec w, const float* __restrict__ state, const int* __restrict__ positions,
                                    const int* __restrict__ row_entry, const int* __restrict__ entry_slots,
-                                   int channels, int taps, int add_input, int act) {
+                                   int channels, int taps, int add_input, int act, float* __restrict__ own_state) {
     const int c = blockIdx.y * blockDim.x + threadIdx.x;
     const int r = blockIdx.x;
     if (c >= channels) return;
@@ -110,8 +142,14 @@ __global__ void causal_conv_kernel(const TIn* __restrict__ in, long in_stride, T
         else h = mine[static_cast<long>(taps - 1 - (back - inside)) * channels];
         acc = fmaf(load_any(w, static_cast<long>(c) * taps + (taps - 1 - back)), h, acc);
     }
-    if (add_input) acc += to_float(in[static_cast<long>(r) * in_stride + c]);
+    const float now = to_float(in[static_cast<long>(r) * in_stride + c]);
+    if (add_input) acc += now;
     out[static_cast<long>(r) * out_stride + c] = from_float<TOut>(activate(acc, act));
+    if (own_state) {      // a step of single rows, every row another request: this thread alone touches (slot, channel)
+        float* keep = own_state + (static_cast<long>(entry_slots[e]) * (taps - 1)) * channels + c;
+        for (int j = 0; j + 2 < taps; ++j) keep[static_cast<long>(j) * channels] = pos - (taps - 2 - j) < 0 ? 0.f : keep[static_cast<long>(j + 1) * channels];
+        keep[static_cast<long>(taps - 2) * channels] = now;
+    }
 }
 
 template <typename TIn>
@@ -147,19 +185,31 @@ __global__ void head_norm_gate_kernel(const float* __restrict__ o, const float* 
     const float* src = o + at * vdim;
     float under = 1.f;
     if (dot) under = fmaxf(fabsf(dot[at]), expf(-top[at])) + 1e-6f;
+    constexpr int kKept = 8;                                   // values a lane keeps between the two passes
+    float kept[kKept];
     float ss = 0.f;
-    for (int j = lane; j < vdim; j += kWave) {
+#pragma unroll
+    for (int n = 0; n < kKept; ++n) {
+        const int j = lane + n * kWave;
+        kept[n] = j < vdim ? src[j] / under : 0.f;
+        ss = fmaf(kept[n], kept[n], ss);
+    }
+    for (int j = lane + kKept * kWave; j < vdim; j += kWave) {
         const float v = src[j] / under;
         ss = fmaf(v, v, ss);
     }
     const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(vdim) + eps);
     TOut* dst = out + at * vdim;
-    for (int j = lane; j < vdim; j += kWave) {
-        float v = (src[j] / under) * inv;
+    auto finish = [&](int j, float v) {
+        v *= inv;
         if (gain.ptr) v *= load_any(gain, gain_per_head ? static_cast<long>(head) * vdim + j : j);
         if (gate) v *= activate(gate[static_cast<long>(row) * gate_stride + static_cast<long>(head) * vdim + j], act);
         dst[j] = from_float<TOut>(v);
-    }
+    };
+#pragma unroll
+    for (int n = 0; n < kKept; ++n)
+        if (lane + n * kWave < vdim) finish(lane + n * kWave, kept[n]);
+    for (int j = lane + kKept * kWave; j < vdim; j += kWave) finish(j, src[j] / under);
 }
 
 constexpr int kMaxBranches = 4;
@@ -212,7 +262,12 @@ using namespace leone;
 
 extern "C" int leone_add_layernorm(float* x, const float* delta, const void* dw, const void* db, float deps,
                                    const void* w, const void* b, int w_dtype, float eps, void* y, int y_dtype,
-                                   const int* rows, int n_out, int hidden, hipStream_t stream) {
+                                   const int* rows, int n_out, int hidden, const void* conv, int conv_dtype, int taps,
+                                   float* conv_state, int write_state, const int* positions, const int* row_entry,
+                                   const int* entry_slots, hipStream_t stream) {
+    LEONE_REQUIRE(!conv || (y && !rows && conv_state && positions && row_entry && entry_slots && taps >= 2 && taps <= kMaxTaps &&
+                            known(conv_dtype)), "add_layernorm: a folded convolution needs its state, the rows' places and 2..%d taps", kMaxTaps);
+    const AnyVec vconv{conv, conv_dtype};
     LEONE_REQUIRE(x && n_out > 0 && hidden > 0, "add_layernorm: needs a stream and positive sizes");
     LEONE_REQUIRE(known(w_dtype) && known(y_dtype), "add_layernorm: unknown element type");
     LEONE_REQUIRE((dw == nullptr) == (db == nullptr), "add_layernorm: the delta's gain and bias come together");
@@ -221,13 +276,16 @@ extern "C" int leone_add_layernorm(float* x, const float* delta, const void* dw,
     LEONE_REQUIRE(y || (delta && !rows), "add_layernorm: nothing to do");
     LEONE_REQUIRE(static_cast<size_t>(hidden) * sizeof(float) <= 64 * 1024, "add_layernorm: rows of %d elements are too long", hidden);
     const AnyVec vdw{dw, w_dtype}, vdb{db, w_dtype}, vw{w, w_dtype}, vb{b, w_dtype};
-    const size_t shared = static_cast<size_t>(hidden) * sizeof(float);
+    const int stage_delta = (delta && static_cast<size_t>(hidden) * 2 * sizeof(float) <= 64 * 1024) ? 1 : 0;
+    const size_t shared = static_cast<size_t>(hidden) * sizeof(float) * (stage_delta ? 2 : 1);
     if (y_dtype == kF32)
         add_layernorm_kernel<float><<<n_out, kNormThreads, shared, stream>>>(x, delta, vdw, vdb, deps, vw, vb, eps,
-                                                                            static_cast<float*>(y), rows, hidden);
+                                                                            static_cast<float*>(y), rows, hidden, vconv, taps,
+                                                                            conv_state, write_state, positions, row_entry, entry_slots, stage_delta);
     else
         add_layernorm_kernel<bf16_t><<<n_out, kNormThreads, shared, stream>>>(x, delta, vdw, vdb, deps, vw, vb, eps,
-                                                                             static_cast<bf16_t*>(y), rows, hidden);
+                                                                             static_cast<bf16_t*>(y), rows, hidden, vconv, taps,
+                                                                             conv_state, write_state, positions, row_entry, entry_slots, stage_delta);
     LEONE_LAUNCH_CHECK("add_layernorm");
     return 0;
 }
@@ -243,27 +301,29 @@ extern "C" int leone_entry_spans(const int* row_entry, const int* positions, con
 extern "C" int leone_causal_conv(const void* in, int in_dtype, long in_stride, void* out, int out_dtype, long out_stride,
                                  const void* w, int w_dtype, float* state, int write_state, const int* spans, int entries,
                                  const int* positions, const int* row_entry, const int* entry_slots, int rows,
-                                 int channels, int taps, int add_input, int act, hipStream_t stream) {
+                                 int channels, int taps, int add_input, int act, int single_rows, hipStream_t stream) {
     LEONE_REQUIRE(in && out && w && state && positions && row_entry && entry_slots, "causal_conv: null pointer");
     LEONE_REQUIRE(known(in_dtype) && known(out_dtype) && known(w_dtype), "causal_conv: unknown element type");
     LEONE_REQUIRE(rows > 0 && channels > 0 && ceil_div(channels, 256) <= 65535 && in_stride >= channels && out_stride >= channels,
                   "causal_conv: %d rows of %d channels", rows, channels);
     LEONE_REQUIRE(taps >= 2 && taps <= kMaxTaps, "causal_conv: %d taps, the kernel takes 2..%d", taps, kMaxTaps);
     LEONE_REQUIRE(act >= kActNone && act <= kActSilu, "causal_conv: unknown activation %d", act);
-    LEONE_REQUIRE(!write_state || (spans && entries > 0 && entries <= 65535), "causal_conv: the state's update needs the entries' spans");
+    LEONE_REQUIRE(!write_state || single_rows || (spans && entries > 0 && entries <= 65535),
+                  "causal_conv: the state's update needs the entries' spans");
     const AnyVec vw{w, w_dtype};
     const dim3 grid(rows, ceil_div(channels, 256));
 #define LEONE_CONV(TIN, TOUT)                                                                                         \
     causal_conv_kernel<TIN, TOUT><<<grid, 256, 0, stream>>>(static_cast<const TIN*>(in), in_stride, static_cast<TOUT*>(out), \
                                                             out_stride, vw, state, positions, row_entry, entry_slots, \
-                                                            channels, taps, add_input, act)
+                                                            channels, taps, add_input, act,                          \
+                                                            (write_state && single_rows) ? state : nullptr)
     if (in_dtype == kF32 && out_dtype == kF32) LEONE_CONV(float, float);
     else if (in_dtype == kF32) LEONE_CONV(float, bf16_t);
     else if (out_dtype == kF32) LEONE_CONV(bf16_t, float);
     else LEONE_CONV(bf16_t, bf16_t);
 #undef LEONE_CONV
     LEONE_LAUNCH_CHECK("causal_conv");
-    if (write_state) {
+    if (write_state && !single_rows) {
         const dim3 sgrid(ceil_div(channels, 256), entries);
         if (in_dtype == kF32)
             causal_conv_state_kernel<float><<<sgrid, 256, 0, stream>>>(static_cast<const float*>(in), in_stride, state, spans,

@@ -202,21 +202,25 @@ int leone_sample_truncated(const float* logits, const double* params, int* out, 
 
 // ---- layers that keep state of their own per request (layernorm_conv.hip, recurrent.hip) ----------------------
 // x += LayerNorm(delta; dw, db, deps) if delta comes (dw null: added as it is), then y = LayerNorm(x; w, b, eps)
-// if y is wanted.  With `rows` (indices) row i of y comes from row rows[i] and x is not written.
+// if y is wanted.  With `rows` (indices) row i of y comes from row rows[i] and x is not written.  With `conv`
+// ([hidden, taps]; a step of single rows, every row another request) y is h + conv(h) over the request's last
+// inputs in conv_state [slots, taps - 1, hidden], which this row then joins (see leone_causal_conv).
 int leone_add_layernorm(float* x, const float* delta, const void* dw, const void* db, float deps, const void* w,
                         const void* b, int w_dtype, float eps, void* y, int y_dtype, const int* rows, int n_out,
-                        int hidden, hipStream_t stream);
+                        int hidden, const void* conv, int conv_dtype, int taps, float* conv_state, int write_state,
+                        const int* positions, const int* row_entry, const int* entry_slots, hipStream_t stream);
 // spans[4e .. 4e + 3]: first row and end of entry e (an entry's rows are consecutive), the state slot it reads
 // (-1 at a sequence's start: zeros) and the one it writes.
 int leone_entry_spans(const int* row_entry, const int* positions, const int* entry_slots, int rows, int* spans,
                       hipStream_t stream);
 // A causal convolution over time per channel, w [channels, taps] with the last tap on the current row; the
 // rows before a portion come from state [slots, taps - 1, channels] (float), which is brought up to date if asked.
-// act: 0 none, 1 sigmoid, 2 silu.
+// act: 0 none, 1 sigmoid, 2 silu.  single_rows: every entry brings one row, and the kernel that convolves moves the
+// state on as well (otherwise a second launch does, from the entries' spans).
 int leone_causal_conv(const void* in, int in_dtype, long in_stride, void* out, int out_dtype, long out_stride,
                       const void* w, int w_dtype, float* state, int write_state, const int* spans, int entries,
                       const int* positions, const int* row_entry, const int* entry_slots, int rows, int channels,
-                      int taps, int add_input, int act, hipStream_t stream);
+                      int taps, int add_input, int act, int single_rows, hipStream_t stream);
 // out = (o / (max(|dot|, exp(-top)) + 1e-6) if dot comes) / rms over vdim * gain * act(gate), head by head.
 int leone_head_norm_gate(const float* o, const float* dot, const float* top, const void* gain, int gain_dtype,
                          int gain_per_head, const float* gate, long gate_stride, int act, float eps, void* out,

@@ -382,14 +382,18 @@ class Engine:
                     or tuple(device_tokens.shape) != (len(entries),)):
                 raise StepError(f"device tokens must be int32 [{len(entries)}] on {self.device}")
         self.poison_freed_pages()              # what a scheduler on the same manager has freed since the last step
-        # A failed step gives its pages back (rollback) and leaves per-request state as it found it.
-        saved_state = self.pools.snapshot_state([self.cache.slot(e.request) for e in entries])
+        # A failed step gives its pages back (rollback) and leaves per-request state as it found it.  A step that is
+        # replayed from a recording it already has cannot fail half way (it is refused before the replay or not at
+        # all), so the copy of the state, a kernel for every state tensor of the model, is left out there.
+        replayed = self.graphs and not profile.recording() and all(len(e.tokens) == 1 for e in entries)
+        saved_state = None if (replayed and self._has_recording(entries)) else \
+            self.pools.snapshot_state([self.cache.slot(e.request) for e in entries])
         try:
             for e in entries:
                 if self.cache.length(e.request) == 0:
                     self.pools.zero_state(self.cache.slot(e.request))   # a request's state starts from zero
             # A step that is being profiled runs call by call: a replayed recording has no calls to time.
-            if self.graphs and not profile.recording() and all(len(e.tokens) == 1 for e in entries):
+            if replayed:
                 logits, rows = self._run_decode_graph(entries, device_tokens)
             else:
                 tokens, context, rows = self._build_context(entries)
@@ -409,6 +413,14 @@ class Engine:
             self.cache.commit(e.request, len(e.tokens))
         self.poison_freed_pages()              # pages a window has passed
         return StepOutput(logits, rows)
+
+    def _has_recording(self, entries: Sequence[StepEntry]) -> bool:
+        """Whether a step of one token for each of these requests would be replayed from a recording made earlier."""
+        state = self._decode_graphs.get(len(entries))
+        if state is None:
+            return False
+        positions = max(self.cache.length(e.request) for e in entries) + 1
+        return context_bucket(positions, self.max_context) in state.recordings
 
     def _run_decode_graph(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None):
         """One decoded token for each entry, replayed from the recording for this batch size."""

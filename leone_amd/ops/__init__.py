@@ -1090,10 +1090,13 @@ class NormedDelta:
 
 def add_layernorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional[torch.Tensor],
                   bias: Optional[torch.Tensor], eps: float, out_dtype: Optional[torch.dtype],
-                  rows: Optional[torch.Tensor] = None, delta_norm: Optional[tuple] = None) -> Optional[torch.Tensor]:
+                  rows: Optional[torch.Tensor] = None, delta_norm: Optional[tuple] = None,
+                  conv: Optional[tuple] = None) -> Optional[torch.Tensor]:
     """x += delta, where ``delta_norm`` = (gain, bias, eps) says that the delta goes through a layer norm of its
     own first; then y = (x - mean) / sqrt(var + eps) * gain + bias in ``out_dtype`` (None: no y, only the sum).
-    With ``rows`` y[i] comes from row rows[i] and x is not written.  Means and variances are float."""
+    With ``rows`` y[i] comes from row rows[i] and x is not written.  Means and variances are float.
+    ``conv`` = (weight ``[hidden, taps]``, state, step, write_state), for a step of single rows only: what comes
+    out is y + conv(y) as ``causal_conv(add_input=True)`` gives it, and the state has moved on, in the same launch."""
     n, hidden = x.shape
     n_out = n if rows is None else rows.numel()
     if delta is not None and delta.dtype != torch.float32:
@@ -1109,8 +1112,23 @@ def add_layernorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional
          _dev(gain, "gain", None, (hidden,)), _dev(bias, "bias", None, (hidden,)),
          _code(vectors[0], "gain") if vectors else F32, float(eps), _dev(y, "normed rows"),
          _CODES[out_dtype] if out_dtype is not None else F32,
-         _dev(rows, "rows", torch.int32) if rows is not None else 0, n_out, hidden, _stream())
+         _dev(rows, "rows", torch.int32) if rows is not None else 0, n_out, hidden, *_folded_conv(conv, n, hidden), _stream())
     return y
+
+
+def _folded_conv(conv, rows: int, hidden: int) -> tuple:
+    """The arguments of a convolution folded into ``add_layernorm``."""
+    if conv is None:
+        return 0, F32, 0, 0, 0, 0, 0, 0
+    weight, state, step, write_state = conv
+    taps = weight.shape[1]
+    if not step.decode_only or step.rows != rows:
+        raise KernelError("add_layernorm: a convolution is folded in only for a step of single rows")
+    if tuple(weight.shape) != (hidden, taps) or state.dtype != torch.float32 or tuple(state.shape[1:]) != (taps - 1, hidden):
+        raise KernelError(f"add_layernorm: conv weight {tuple(weight.shape)} and state {tuple(state.shape)} do not fit rows of {hidden}")
+    return (_dev(weight, "conv weight"), _code(weight, "conv weight"), taps, _dev(state, "conv state"), 1 if write_state else 0,
+            _dev(step.positions, "positions", torch.int32, (rows,)), _dev(step.row_entry, "row map", torch.int32, (rows,)),
+            _dev(step.entry_slots, "slots", torch.int32))
 
 
 def entry_spans(step) -> torch.Tensor:
@@ -1182,12 +1200,13 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, step
         raise KernelError("causal_conv: tensor is not on the GPU")
     out = torch.empty((rows, channels), dtype=out_dtype, device=x.device)
     spans = entry_spans(step)
+    single_rows = bool(step.decode_only) and step.entry_slots.numel() == rows
     call("leone_causal_conv", x.data_ptr(), _code(x, "conv input"), x.stride(0), _dev(out, "conv out"), _CODES[out_dtype],
          channels, _dev(weight, "conv weight"), _code(weight, "conv weight"), _dev(state, "conv state"),
          1 if write_state else 0, _dev(spans, "spans"), spans.shape[0],
          _dev(step.positions, "positions", torch.int32, (rows,)), _dev(step.row_entry, "row map", torch.int32, (rows,)),
          _dev(step.entry_slots, "slots", torch.int32), rows, channels, taps, 1 if add_input else 0,
-         ACTIVATIONS[activation], _stream())
+         ACTIVATIONS[activation], 1 if single_rows else 0, _stream())
     return out
 
 

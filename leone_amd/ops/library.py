@@ -52,10 +52,11 @@ _PROTOTYPES = {
     "leone_sample_temperature": [P, P, P, P, P, P, P, P, c_int, c_int, P],
     "leone_top_candidates": [P, P, P, P, c_int, c_int, c_int, P],
     "leone_sample_truncated": [P, P, P, c_int, c_int, P],
-    "leone_add_layernorm": [P, P, P, P, c_float, P, P, c_int, c_float, P, c_int, P, c_int, c_int, P],
+    "leone_add_layernorm": [P, P, P, P, c_float, P, P, c_int, c_float, P, c_int, P, c_int, c_int, P, c_int, c_int, P, c_int,
+                            P, P, P, P],
     "leone_entry_spans": [P, P, P, c_int, P, P],
     "leone_causal_conv": [P, c_int, ctypes.c_long, P, c_int, ctypes.c_long, P, c_int, P, c_int, P, c_int, P, P, P, c_int,
-                          c_int, c_int, c_int, c_int, P],
+                          c_int, c_int, c_int, c_int, c_int, P],
     "leone_head_norm_gate": [P, P, P, P, c_int, c_int, P, ctypes.c_long, c_int, c_float, P, c_int, c_int, c_int, c_int, P],
     "leone_rms_mix": [P, P, c_int, c_int, c_float, c_float, P, c_int, c_int, P],
     "leone_relu_squared": [P, P, c_int, ctypes.c_long, P],

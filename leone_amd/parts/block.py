@@ -159,6 +159,9 @@ class SandwichBlock(Part):
         convolution if there is one."""
         if conv is None:
             return norm.add_norm(x, pending, step.dtype)
+        if step.decode_only and getattr(norm, "folds_conv", False) and conv.add_input and conv.activation is None:
+            # single decoded tokens: norm, convolution and the move of its state in one launch
+            return norm.add_norm(x, pending, step.dtype, conv=(conv.weight, cache.state, step, cache.writes))
         return conv.forward(norm.add_norm(x, pending, torch.float32), step, cache, step.dtype)
 
     def forward(self, x: torch.Tensor, pending, step: StepContext, cache):

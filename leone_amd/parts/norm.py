@@ -59,6 +59,8 @@ class RmsNorm(Part):
 
 @NORMS.register("layernorm")
 class LayerNorm(Part):
+    folds_conv = True      # add_norm(..., conv=) takes the residual-form convolution of single rows into its kernel
+
     """y = (x - mean) / sqrt(var + eps) * weight + bias, var the mean squared deviation; mean and variance in float.
 
     Parameters: ``size``, ``eps``, ``weight``, ``bias`` (tensor names).  ``add_norm`` also takes a delta that
@@ -84,7 +86,10 @@ class LayerNorm(Part):
         if self.gain.dtype != self.bias.dtype:
             self.gain, self.bias = self.gain.float(), self.bias.float()
 
-    def add_norm(self, x: torch.Tensor, delta, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def add_norm(self, x: torch.Tensor, delta, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                 conv: Optional[tuple] = None) -> torch.Tensor:
+        """``conv`` = (weight, state, step, write_state): in a step of single rows the input convolution of the
+        sublayer that reads this norm is done in the same kernel (``ops.add_layernorm``)."""
         if isinstance(delta, ops.PreparedRows):
             delta = None
         delta_norm = None
@@ -96,7 +101,7 @@ class LayerNorm(Part):
                 delta = delta.materialize()
         elif delta is not None and delta.dim() == 3:
             delta = delta.sum(dim=0)          # planes of a product cut along its inner dimension
-        return ops.add_layernorm(x, delta, self.gain, self.bias, self.eps, out_dtype, rows, delta_norm)
+        return ops.add_layernorm(x, delta, self.gain, self.bias, self.eps, out_dtype, rows, delta_norm, conv)
 
     def apply(self, rows: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
         """The norm of float32 rows that are no stream (nothing is added, nothing written back)."""
