@@ -26,6 +26,7 @@ namespace leone {
 constexpr int kScanTokens = 16;
 constexpr int kLaneRows = 32;       // key channels a lane holds
 constexpr int kScanThreads = 256;
+constexpr int kLaneCols = 2;        // columns a lane holds in the outer-product scan: every q and k it reads serves both
 
 // Over how many lanes a column of `dim` key channels is spread: 1, 2, 4 or 8 (dim up to 256).
 inline int lane_groups(int dim) { return dim <= 32 ? 1 : dim <= 64 ? 2 : dim <= 128 ? 4 : 8; }
@@ -144,24 +145,33 @@ __global__ void __launch_bounds__(kScanThreads) outer_scan_kernel(OuterScanArgs 
     float* sb = sa + kScanTokens;
     const int head = blockIdx.y, tid = threadIdx.x, lane = tid % kWave;
     const Segment seg = p.segments[blockIdx.x];
-    const int per_wave = kWave / groups;                       // columns a wave
-    const int part = lane / per_wave;                          // which 32 key channels of the column this lane holds
-    const int col = (blockIdx.z * (kScanThreads / kWave) + tid / kWave) * per_wave + lane % per_wave;
+    const int per_wave = kWave / groups;                       // lanes a wave has for columns; each holds kLaneCols of them
+    const int part = lane / per_wave;                          // which 32 key channels of its columns this lane holds
     const int cols = p.vdim + (p.norm_column ? 1 : 0);
-    const bool is_value = col < p.vdim, is_norm = p.norm_column && col == p.vdim;
+    int col[kLaneCols];
+    bool is_value[kLaneCols], is_norm[kLaneCols];
+#pragma unroll
+    for (int c = 0; c < kLaneCols; ++c) {
+        col[c] = ((blockIdx.z * (kScanThreads / kWave) + tid / kWave) * kLaneCols + c) * per_wave + lane % per_wave;
+        is_value[c] = col[c] < p.vdim;
+        is_norm[c] = p.norm_column && col[c] == p.vdim;
+    }
     const int first = seg.first, n = seg.end - seg.first;
     const int ch0 = part * kLaneRows;
     const float* from = seg.in < 0 ? nullptr : p.state_in + seg.in * p.in_stride + head * p.head_stride;
 
-    float S[kLaneRows];
+    float S[kLaneCols][kLaneRows];
 #pragma unroll
-    for (int i = 0; i < kLaneRows; ++i) {
-        float v = 0.f;
-        if (from && ch0 + i < p.dim) {
-            if (is_value) v = from[static_cast<long>(ch0 + i) * p.vdim + col];
-            else if (is_norm) v = from[static_cast<long>(p.dim) * p.vdim + ch0 + i];
+    for (int c = 0; c < kLaneCols; ++c) {
+#pragma unroll
+        for (int i = 0; i < kLaneRows; ++i) {
+            float v = 0.f;
+            if (from && ch0 + i < p.dim) {
+                if (is_value[c]) v = from[static_cast<long>(ch0 + i) * p.vdim + col[c]];
+                else if (is_norm[c]) v = from[static_cast<long>(p.dim) * p.vdim + ch0 + i];
+            }
+            S[c][i] = v;
         }
-        S[i] = v;
     }
     const float fixed = p.coef ? 0.f : p.decay[head];
     float carried = 1.f;                                      // the product of the segment's decays
@@ -189,39 +199,69 @@ __global__ void __launch_bounds__(kScanThreads) outer_scan_kernel(OuterScanArgs 
             sb[tid] = p.no_input ? 0.f : (p.coef ? p.coef[2 * at + 1] : 1.f);
         }
         __syncthreads();
-        if (col < cols) {                                      // the lanes of a column are in or out together
+        if (col[0] < cols) {                                   // the lanes of a column are in or out together
             for (int t = 0; t < here; ++t) {
                 const long row = first + t0 + t;
                 const float a = sa[t];
-                const float v = (is_value && !p.no_input) ? p.proj[row * p.stride + p.v_off + head * p.vdim + col] : 1.f;
-                const float bv = sb[t] * v;
                 const float* kt = sk + t * dkp + ch0;
                 const float* qt = sq + t * dkp + ch0;
-                float acc = 0.f;
+                float acc[kLaneCols];
+                if (p.no_input) {                              // nothing is written: the state decays and is read
 #pragma unroll
-                for (int i = 0; i < kLaneRows; ++i) {
-                    S[i] = fmaf(a, S[i], kt[i] * bv);
-                    acc = fmaf(S[i], qt[i], acc);
+                    for (int c = 0; c < kLaneCols; ++c) acc[c] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < kLaneRows; ++i) {
+                        const float q = qt[i];
+#pragma unroll
+                        for (int c = 0; c < kLaneCols; ++c) {
+                            S[c][i] *= a;
+                            acc[c] = fmaf(S[c][i], q, acc[c]);
+                        }
+                    }
+                } else {
+                    float bv[kLaneCols];
+#pragma unroll
+                    for (int c = 0; c < kLaneCols; ++c) {
+                        const float v = is_value[c] ? p.proj[row * p.stride + p.v_off + head * p.vdim + col[c]] : 1.f;
+                        bv[c] = sb[t] * v;
+                        acc[c] = 0.f;
+                    }
+#pragma unroll
+                    for (int i = 0; i < kLaneRows; ++i) {
+                        const float k = kt[i], q = qt[i];
+#pragma unroll
+                        for (int c = 0; c < kLaneCols; ++c) {
+                            S[c][i] = fmaf(a, S[c][i], k * bv[c]);
+                            acc[c] = fmaf(S[c][i], q, acc[c]);
+                        }
+                    }
                 }
-                for (int off = per_wave; off < kWave; off <<= 1) acc += __shfl_xor(acc, off, kWave);
                 carried *= a;
-                if (part == 0) {
-                    const long at = row * p.heads + head;
-                    float* dst = is_value ? p.out + at * p.vdim + col : p.dot + at;
-                    *dst = p.accumulate ? *dst + acc : acc;
+#pragma unroll
+                for (int c = 0; c < kLaneCols; ++c) {
+                    for (int off = per_wave; off < kWave; off <<= 1) acc[c] += __shfl_xor(acc[c], off, kWave);
+                    if (part == 0 && col[c] < cols) {
+                        const long at = row * p.heads + head;
+                        float* dst = is_value[c] ? p.out + at * p.vdim + col[c] : p.dot + at;
+                        *dst = p.accumulate ? *dst + acc[c] : acc[c];
+                    }
                 }
             }
         }
         __syncthreads();
     }
     if (p.decay_product && blockIdx.z == 0 && tid == 0) p.decay_product[static_cast<long>(blockIdx.x) * p.heads + head] = carried;
-    if (!p.state_out || seg.out < 0 || col >= cols) return;
+    if (!p.state_out || seg.out < 0) return;
     float* to = p.state_out + seg.out * p.out_stride + head * p.head_stride;
 #pragma unroll
-    for (int i = 0; i < kLaneRows; ++i) {
-        if (ch0 + i < p.dim) {
-            if (is_value) to[static_cast<long>(ch0 + i) * p.vdim + col] = S[i];
-            else to[static_cast<long>(p.dim) * p.vdim + ch0 + i] = S[i];
+    for (int c = 0; c < kLaneCols; ++c) {
+        if (col[c] >= cols) continue;
+#pragma unroll
+        for (int i = 0; i < kLaneRows; ++i) {
+            if (ch0 + i < p.dim) {
+                if (is_value[c]) to[static_cast<long>(ch0 + i) * p.vdim + col[c]] = S[c][i];
+                else to[static_cast<long>(p.dim) * p.vdim + ch0 + i] = S[c][i];
+            }
         }
     }
 }
@@ -484,7 +524,7 @@ extern "C" int leone_outer_scan(const float* proj, long stride, int q_off, int k
                     reinterpret_cast<const Segment*>(segments), state_in, in_stride, state_out, out_stride, head_stride,
                     decay_product, out, dot, heads, dim, vdim};
     const int groups = lane_groups(dim);
-    const int per_block = (kScanThreads / kWave) * (kWave / groups);          // columns a workgroup
+    const int per_block = (kScanThreads / kWave) * (kWave / groups) * kLaneCols;          // columns a workgroup
     const dim3 grid(n_segments, heads, ceil_div(vdim + (norm_column ? 1 : 0), per_block));
     const size_t shared = (2 * kScanTokens * groups * kLaneRows + 2 * kScanTokens) * sizeof(float);
     outer_scan_kernel<<<grid, kScanThreads, shared, stream>>>(a, groups);
