@@ -350,6 +350,7 @@ def run_scenario(name: str, dtype: str = "bfloat16", layers: Optional[int] = Non
 DESIGN_SIZES = {
     "w2048": dict(width=2048, layers=8, vocab=32768, batch=8, context=2048, prompt=2048),
     "w4096": dict(width=4096, layers=8, vocab=32768, batch=8, context=2048, prompt=2048),
+    "w512": dict(width=512, layers=4, vocab=4096, batch=2, context=512, prompt=512),       # small: for a quick look
 }
 
 

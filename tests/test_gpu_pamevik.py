@@ -460,3 +460,26 @@ def test_layer_norm_with_the_norm_behind_a_sublayer_folded_in():
     stream = x.to(DEV)
     picked = norms["b"].add_norm(stream, ops.NormedDelta(delta.to(DEV), norms["a"]), torch.float32, rows=rows)
     assert (picked.cpu().double() - want[[5, 0, 5]]).abs().max() < 1e-5 and torch.equal(stream.cpu(), x)
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_feed_forward_and_branch_mix_alone(dtype_name):
+    """down(relu(up y)^2) at sizes off the runs of 8, and the parallel mixer's way of joining its branches: each
+    over its root mean square, times its own gain, half the sum (two stand-in branches that multiply by a matrix)."""
+    from leone_amd import ops
+    from leone_amd.parts import FEED_FORWARDS, PartSpec
+    dtype = DTYPES[dtype_name]
+    gen = torch.Generator().manual_seed(12)
+    up, down = (torch.randn(100, 40, generator=gen) / 6).to(dtype), (torch.randn(40, 100, generator=gen) / 10).to(dtype)
+    part = FEED_FORWARDS.build(PartSpec("relu2", {"hidden": 40, "intermediate": 100, "up": "u", "down": "d"}))
+    part.bind({"u": up.to(DEV), "d": down.to(DEV)})
+    y = torch.randn(21, 40, generator=gen).to(dtype)
+    got = part.forward(y.to(DEV), step_of([(0, i) for i in range(21)], dtype, [0]))
+    want = plain.dense_feed_forward(y.to(plain.F), {"up": up.to(plain.F), "down": down.to(plain.F)}, "")
+    assert got.dtype == torch.float32
+    assert pu.relative_error(got.cpu().numpy(), want.numpy()).max() <= (2e-6 if dtype_name == "float32" else 2e-2)
+    left, right = torch.randn(9, 72, generator=gen) * 3, torch.randn(9, 72, generator=gen) * 0.01
+    gl, gr = (1 + 0.3 * torch.randn(72, generator=gen)).to(dtype), (1 + 0.3 * torch.randn(72, generator=gen)).to(dtype)
+    mixed = ops.rms_mix([left.to(DEV), right.to(DEV)], [gl.to(DEV), gr.to(DEV)], 1e-5, 0.5)
+    want = 0.5 * (plain.unit_rms(left.double(), 1e-5) * gl.double() + plain.unit_rms(right.double(), 1e-5) * gr.double())
+    assert (mixed.cpu().double() - want).abs().max() < 1e-5
