@@ -20,7 +20,7 @@ namespace leone {
 
 constexpr int kRowThreads = 256;
 constexpr int kRowWaves = kRowThreads / kWave;
-constexpr int kRowDimsPerLane = 4;                      // head_dim up to 256
+constexpr int kRowDimsPerLane = 8;                      // keys and values of up to 512 elements a head
 constexpr int kRowMaxHeadDim = kWave * kRowDimsPerLane;
 
 // One block per (row, query head).  Wave w takes keys first + w, first + w + 4,
@@ -55,7 +55,9 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
     }
 
     float m = -INFINITY, l = 0.f;
-    float acc[kRowDimsPerLane] = {0.f, 0.f, 0.f, 0.f};
+    float acc[kRowDimsPerLane];
+#pragma unroll
+    for (int i = 0; i < kRowDimsPerLane; ++i) acc[i] = 0.f;
     for (int j = first + wave; j <= pos; j += kRowWaves) {
         const int page = table[j / page_tokens];
         if (page < 0) {  // an unmapped block: poison the result instead of reading outside the pool

@@ -483,3 +483,23 @@ def test_feed_forward_and_branch_mix_alone(dtype_name):
     mixed = ops.rms_mix([left.to(DEV), right.to(DEV)], [gl.to(DEV), gr.to(DEV)], 1e-5, 0.5)
     want = 0.5 * (plain.unit_rms(left.double(), 1e-5) * gl.double() + plain.unit_rms(right.double(), 1e-5) * gr.double())
     assert (mixed.cpu().double() - want).abs().max() < 1e-5
+
+
+def test_command_line_generates_from_token_ids(tmp_path):
+    """``leone generate`` on a Pamevik folder: greedy tokens as the plain implementation picks them."""
+    from leone_amd import cli
+    raw = pu.SMALL["S"]
+    weights = pu.make_weights(raw, 61, pu.RANKS["S"], torch.float32)
+    folder = pu.write_dir(str(tmp_path / "model"), raw, weights)
+    prompt = [5, 17, 3, 99, 42, 7]
+    out = str(tmp_path / "tokens.json")
+    assert cli.main(["generate", "-m", folder, "--prompt-tokens", ",".join(map(str, prompt)), "-n", "8", "--dtype", "float32",
+                     "--ignore-eos", "--debug-tokens", out]) == 0
+    with open(out) as handle:
+        got = json.load(handle)
+    tokens = list(prompt)
+    for token in got:
+        logits = plain.forward(raw, weights, tokens)[-1]
+        assert token == int(logits.argmax()) or float(logits.max() - logits[token]) < 1e-4
+        tokens.append(token)
+    assert len(got) == 8
