@@ -307,7 +307,8 @@ struct DeltaScanArgs {
     float* state_out;
     long out_stride;
     float* transition;          // [segments, heads, dim, dim] or null: what the segment's rows do to a state that comes
-                                // in, as a matrix: dim more columns that start as the unit vectors and are given v = 0
+                                // in, as a matrix: dim more columns that start as the unit vectors and are given v = 0;
+                                // stored [unit vector j][channel i], the order in which the chain reads it
     float* out;                 // [rows, heads, vdim]
     int heads, kv_heads, dim, vdim;
 };
@@ -347,26 +348,35 @@ __global__ void __launch_bounds__(kScanThreads) delta_scan_kernel(DeltaScanArgs 
 
     for (int t0 = 0; t0 < n; t0 += kScanTokens) {
         const int here = min(kScanTokens, n - t0);
-        for (int t = wave; t < here; t += kScanThreads / kWave) {       // a wave prepares a token's vectors
-            const long row = first + t0 + t;
-            const float* base = p.qkv + row * p.stride;
-            const float* qs = base + p.q_off + kvh * p.dim;
-            const float* ks = base + p.k_off + kvh * p.dim;
-            float qq = 0.f, kk = 0.f;
-            for (int i = lane; i < p.dim; i += kWave) {
-                qq = fmaf(qs[i], qs[i], qq);
-                kk = fmaf(ks[i], ks[i], kk);
+        {   // sixteen lanes prepare a row's vectors, all rows of the chunk at once
+            constexpr int kRowLanes = kScanThreads / kScanTokens;
+            const int t = tid / kRowLanes, sub = tid % kRowLanes;
+            if (t < here) {
+                const long row = first + t0 + t;
+                const float* base = p.qkv + row * p.stride;
+                const float* qs = base + p.q_off + kvh * p.dim;
+                const float* ks = base + p.k_off + kvh * p.dim;
+                float qq = 0.f, kk = 0.f;
+                for (int i = sub; i < p.dim; i += kRowLanes) {
+                    qq = fmaf(qs[i], qs[i], qq);
+                    kk = fmaf(ks[i], ks[i], kk);
+                }
+#pragma unroll
+                for (int off = kRowLanes / 2; off > 0; off >>= 1) {
+                    qq += __shfl_xor(qq, off, kWave);
+                    kk += __shfl_xor(kk, off, kWave);
+                }
+                const float qinv = p.q_scale / sqrtf(qq + p.unit_eps);
+                const float kinv = 1.0f / sqrtf(kk + p.unit_eps);
+                for (int i = sub; i < dkp; i += kRowLanes) {
+                    const bool in = i < p.dim;
+                    sq[t * dkp + i] = in ? qs[i] * qinv : 0.f;
+                    sk[t * dkp + i] = in ? ks[i] * kinv : 0.f;
+                    const long ch = static_cast<long>(head) * p.dim + i;
+                    sg[t * dkp + i] = in ? expf(-rate * softplus_f(p.step[row * p.step_stride + ch] + load_any(p.step_bias, ch))) : 1.f;
+                }
+                if (sub == 0) sbeta[t] = 1.0f / (1.0f + expf(-p.beta[row * p.beta_stride + head]));
             }
-            const float qinv = p.q_scale / sqrtf(wave_sum(qq) + p.unit_eps);
-            const float kinv = 1.0f / sqrtf(wave_sum(kk) + p.unit_eps);
-            for (int i = lane; i < dkp; i += kWave) {
-                const bool in = i < p.dim;
-                sq[t * dkp + i] = in ? qs[i] * qinv : 0.f;
-                sk[t * dkp + i] = in ? ks[i] * kinv : 0.f;
-                const long ch = static_cast<long>(head) * p.dim + i;
-                sg[t * dkp + i] = in ? expf(-rate * softplus_f(p.step[row * p.step_stride + ch] + load_any(p.step_bias, ch))) : 1.f;
-            }
-            if (lane == 0) sbeta[t] = 1.0f / (1.0f + expf(-p.beta[row * p.beta_stride + head]));
         }
         __syncthreads();
         if (live) {                                            // the lanes of a column are in or out together
@@ -403,7 +413,7 @@ __global__ void __launch_bounds__(kScanThreads) delta_scan_kernel(DeltaScanArgs 
         float* to = p.transition + (static_cast<long>(blockIdx.x) * p.heads + head) * p.dim * p.dim;
 #pragma unroll
         for (int i = 0; i < kLaneRows; ++i)
-            if (ch0 + i < p.dim) to[static_cast<long>(ch0 + i) * p.dim + unit] = S[i];
+            if (ch0 + i < p.dim) to[static_cast<long>(unit) * p.dim + ch0 + i] = S[i];
         return;
     }
     if (!p.state_out || seg.out < 0 || !is_value) return;
@@ -452,8 +462,8 @@ delta_chain_kernel(const int* __restrict__ links, float* __restrict__ work, long
         for (int j0 = 0; j0 < dim; j0 += tile) {
             __syncthreads();
             for (int idx = tid; idx < tile * dkp; idx += kScanThreads) {
-                const int jj = idx % tile, i = idx / tile;
-                sT[jj * dkp + i] = (i < dim && j0 + jj < dim) ? T[static_cast<long>(i) * dim + j0 + jj] : 0.f;
+                const int jj = idx / dkp, i = idx % dkp;
+                sT[idx] = (i < dim && j0 + jj < dim) ? T[static_cast<long>(j0 + jj) * dim + i] : 0.f;
             }
             __syncthreads();
             const int width = min(tile, dim - j0);
