@@ -27,7 +27,8 @@ DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 # key, a lost state, a tap off by one) is of the logits' own size at many positions.
 TOLERANCE = {"float32": 3e-5, "bfloat16": 4e-2}
 OUTLIER = {"float32": 1.0, "bfloat16": 7.5}
-LENGTHS = {"P": [1, 2, 37, 130, 64, 9], "Q": [70, 3, 150, 33, 81], "R": [90, 17, 65, 2, 48], "S": [5, 100, 31, 66, 12]}
+LENGTHS = {"P": [1, 2, 37, 130, 64, 9], "Q": [70, 3, 150, 33, 81], "R": [90, 17, 65, 2, 48], "S": [5, 100, 31, 66, 12],
+           "T": [140, 20, 75, 1, 50]}
 
 
 def widened(weights):
@@ -503,3 +504,18 @@ def test_command_line_generates_from_token_ids(tmp_path):
         assert token == int(logits.argmax()) or float(logits.max() - logits[token]) < 1e-4
         tokens.append(token)
     assert len(got) == 8
+
+
+def test_which_attention_kernels_a_branch_gets(cases):
+    """Values of another size than the keys go to the row kernel; keys and values of one size that the matrix-core
+    kernels take go to them in bfloat16 (the gate is applied behind them), and to the row kernel in float32."""
+    folder, _, _ = cases("T", "bfloat16")
+    engine = make_engine(folder, "bfloat16", max_tokens=256)
+    branch = engine.model.layers[0].mixer.branches["left"]
+    assert branch.general and branch.value_dim == branch.head_dim
+    assert branch.attention_kernels(torch.bfloat16, 16, 16) == {"decode": "split_kv", "prompt": "flash"}
+    assert branch.attention_kernels(torch.float32, 16, 16) == {"decode": "rows", "prompt": "rows"}
+    folder, _, _ = cases("P", "bfloat16")
+    other = make_engine(folder, "bfloat16", max_tokens=256).model.layers[1].mixer.branches["left"]
+    assert other.value_dim != other.head_dim
+    assert other.attention_kernels(torch.bfloat16, 16, 16) == {"decode": "rows", "prompt": "rows"}
