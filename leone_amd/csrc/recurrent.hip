@@ -132,8 +132,7 @@ exp_gates_kernel(const float* __restrict__ proj, long stride, int i_off, int f_o
         }
         __syncthreads();
     }
-    const int lane0 = tid;
-    if (write_state && out >= 0 && lane0 == 0) state[out * slot_stride + head * head_stride + top_at] = m;
+    if (write_state && out >= 0 && tid == 0) state[out * slot_stride + head * head_stride + top_at] = m;
 }
 
 __global__ void __launch_bounds__(kScanThreads) outer_scan_kernel(OuterScanArgs p, int groups) {

@@ -8,6 +8,7 @@ from __future__ import annotations
 
 from typing import Optional
 
+import ctypes
 import functools
 import math
 import threading
@@ -1237,7 +1238,6 @@ def head_norm_gate(o: torch.Tensor, heads: int, vdim: int, eps: float, out_dtype
 def rms_mix(branches, gains, eps: float, scale: float) -> torch.Tensor:
     """scale * sum_b rms(branches[b]) * gains[b]: every branch (float32 ``[rows, hidden]``) over its root mean
     square along the row, times its gain."""
-    import ctypes
     rows, hidden = branches[0].shape
     if len(branches) != len(gains) or len({g.dtype for g in gains}) != 1:
         raise KernelError("rms_mix: one gain a branch, all of one type")

@@ -15,9 +15,12 @@ from .context import StepContext
 from .position import rotation_of
 
 
+SCAN_MAX_DIM = 256      # key channels a head may have: 32 a lane over at most 8 lanes (csrc/recurrent.hip)
+
+
 def _check_dim(kind: str, dim: int) -> None:
-    if dim > 256:
-        raise ValueError(f"{kind}: heads of {dim} key channels; the recurrence kernels take up to 256")
+    if dim > SCAN_MAX_DIM:
+        raise ValueError(f"{kind}: heads of {dim} key channels; the recurrence kernels take up to {SCAN_MAX_DIM}")
 
 
 @MIXERS.register("mlstm")
