@@ -18,11 +18,15 @@
 
 namespace leone {
 
-constexpr int kNormThreads = 1024;     // few elements a thread: a row is a handful of trips to memory, not one per element
+// Threads a row.  Few rows (decode steps): 1,024, so that a thread has few elements and a row is a handful of trips to
+// memory, not one per element.  Many rows (prompt portions): 256, so that many rows are in flight on a compute unit.
+constexpr int kNormThreadsFew = 1024;
+constexpr int kNormThreadsMany = 256;
+constexpr int kNormManyRows = 512;
 constexpr int kMaxTaps = 16;
 
 // Mean and inverse deviation of n values read through f(i); every thread gets both.
-template <typename F>
+template <int kNormThreads, typename F>
 __device__ inline void mean_rstd(F value, int n, float eps, float* scratch, float& mean, float& rstd) {
     float s = 0.f;
     for (int i = threadIdx.x; i < n; i += kNormThreads) s += value(i);
@@ -37,7 +41,7 @@ __device__ inline void mean_rstd(F value, int n, float eps, float* scratch, floa
 }
 
 // One workgroup a row; the row lies in shared memory between the passes.
-template <typename TOut>
+template <typename TOut, int kNormThreads>
 __global__ void __launch_bounds__(kNormThreads)
 add_layernorm_kernel(float* __restrict__ x, const float* __restrict__ delta, AnyVec dw, AnyVec db, float deps,
                      AnyVec w, AnyVec b, float eps, TOut* __restrict__ y, const int* __restrict__ rows, int hidden,
@@ -59,8 +63,8 @@ add_layernorm_kernel(float* __restrict__ x, const float* __restrict__ delta, Any
         __syncthreads();
         float mean = 0.f, rstd = 1.f;
         if (dw.ptr) {
-            if (staged) mean_rstd([&](int i) { return staged[i]; }, hidden, deps, scratch, mean, rstd);
-            else mean_rstd([&](int i) { return dr[i]; }, hidden, deps, scratch, mean, rstd);
+            if (staged) mean_rstd<kNormThreads>([&](int i) { return staged[i]; }, hidden, deps, scratch, mean, rstd);
+            else mean_rstd<kNormThreads>([&](int i) { return dr[i]; }, hidden, deps, scratch, mean, rstd);
         }
         for (int i = threadIdx.x; i < hidden; i += kNormThreads) {
             float d = staged ? staged[i] : dr[i];
@@ -75,7 +79,7 @@ add_layernorm_kernel(float* __restrict__ x, const float* __restrict__ delta, Any
     if (!y) return;
     __syncthreads();
     float mean, rstd;
-    mean_rstd([&](int i) { return row_buf[i]; }, hidden, eps, scratch, mean, rstd);
+    mean_rstd<kNormThreads>([&](int i) { return row_buf[i]; }, hidden, eps, scratch, mean, rstd);
     TOut* yr = y + static_cast<long>(blockIdx.x) * hidden;
     if (!conv.ptr) {
         for (int i = threadIdx.x; i < hidden; i += kNormThreads)
@@ -121,34 +125,49 @@ __device__ inline float activate(float v, int act) {
     return act == kActSigmoid ? s : v * s;
 }
 
+constexpr int kConvRows = 8;     // consecutive rows a workgroup takes in a step of many rows: what it must know of a row is
+                                 // fetched once for all of them; a step of few rows has a workgroup a row
+
 template <typename TIn, typename TOut>
 __global__ void causal_conv_kernel(const TIn* __restrict__ in, long in_stride, TOut* __restrict__ out, long out_stride,
                                    AnyVec w, const float* __restrict__ state, const int* __restrict__ positions,
-                                   const int* __restrict__ row_entry, const int* __restrict__ entry_slots,
-                                   int channels, int taps, int add_input, int act, float* __restrict__ own_state) {
+                                   const int* __restrict__ row_entry, const int* __restrict__ entry_slots, int rows,
+                                   int channels, int taps, int add_input, int act, float* __restrict__ own_state, int per_block) {
+    __shared__ int s_inside[kConvRows], s_pos[kConvRows], s_slot[kConvRows];
     const int c = blockIdx.y * blockDim.x + threadIdx.x;
-    const int r = blockIdx.x;
-    if (c >= channels) return;
-    const int e = row_entry[r];
-    const int pos = positions[r];
-    int inside = 0;          // rows of this request that stand before row r in this step, as far as the taps reach
-    while (inside < taps - 1 && r - inside - 1 >= 0 && row_entry[r - inside - 1] == e) ++inside;
-    const float* mine = state + (static_cast<long>(entry_slots[e]) * (taps - 1)) * channels + c;
-    float acc = 0.f;
-    for (int back = taps - 1; back >= 0; --back) {          // oldest input first
-        float h;
-        if (pos - back < 0) h = 0.f;                          // before the sequence's start
-        else if (back <= inside) h = to_float(in[static_cast<long>(r - back) * in_stride + c]);
-        else h = mine[static_cast<long>(taps - 1 - (back - inside)) * channels];
-        acc = fmaf(load_any(w, static_cast<long>(c) * taps + (taps - 1 - back)), h, acc);
+    const int r0 = blockIdx.x * per_block;
+    if (threadIdx.x < per_block && r0 + threadIdx.x < rows) {
+        const int r = r0 + threadIdx.x;
+        const int e = row_entry[r];
+        int inside = 0;      // rows of this request that stand before row r in this step, as far as the taps reach
+        while (inside < taps - 1 && r - inside - 1 >= 0 && row_entry[r - inside - 1] == e) ++inside;
+        s_inside[threadIdx.x] = inside;
+        s_pos[threadIdx.x] = positions[r];
+        s_slot[threadIdx.x] = entry_slots[e];
     }
-    const float now = to_float(in[static_cast<long>(r) * in_stride + c]);
-    if (add_input) acc += now;
-    out[static_cast<long>(r) * out_stride + c] = from_float<TOut>(activate(acc, act));
-    if (own_state) {      // a step of single rows, every row another request: this thread alone touches (slot, channel)
-        float* keep = own_state + (static_cast<long>(entry_slots[e]) * (taps - 1)) * channels + c;
-        for (int j = 0; j + 2 < taps; ++j) keep[static_cast<long>(j) * channels] = pos - (taps - 2 - j) < 0 ? 0.f : keep[static_cast<long>(j + 1) * channels];
-        keep[static_cast<long>(taps - 2) * channels] = now;
+    __syncthreads();
+    if (c >= channels) return;
+    for (int k = 0; k < per_block && r0 + k < rows; ++k) {
+        const int r = r0 + k;
+        const int pos = s_pos[k], inside = s_inside[k];
+        const float* mine = state + (static_cast<long>(s_slot[k]) * (taps - 1)) * channels + c;
+        float acc = 0.f;
+        for (int back = taps - 1; back >= 0; --back) {          // oldest input first
+            float h;
+            if (pos - back < 0) h = 0.f;                          // before the sequence's start
+            else if (back <= inside) h = to_float(in[static_cast<long>(r - back) * in_stride + c]);
+            else h = mine[static_cast<long>(taps - 1 - (back - inside)) * channels];
+            acc = fmaf(load_any(w, static_cast<long>(c) * taps + (taps - 1 - back)), h, acc);
+        }
+        const float now = to_float(in[static_cast<long>(r) * in_stride + c]);
+        if (add_input) acc += now;
+        out[static_cast<long>(r) * out_stride + c] = from_float<TOut>(activate(acc, act));
+        if (own_state) {      // a step of single rows, every row another request: this thread alone touches (slot, channel)
+            float* keep = own_state + (static_cast<long>(s_slot[k]) * (taps - 1)) * channels + c;
+            for (int j = 0; j + 2 < taps; ++j)
+                keep[static_cast<long>(j) * channels] = pos - (taps - 2 - j) < 0 ? 0.f : keep[static_cast<long>(j + 1) * channels];
+            keep[static_cast<long>(taps - 2) * channels] = now;
+        }
     }
 }
 
@@ -218,6 +237,7 @@ struct Branches {
     AnyVec gain[kMaxBranches];
 };
 
+template <int kNormThreads>
 __global__ void __launch_bounds__(kNormThreads)
 rms_mix_kernel(Branches in, int branches, float eps, float scale, float* __restrict__ out, int hidden) {
     __shared__ float scratch[kNormThreads / kWave];
@@ -278,14 +298,19 @@ extern "C" int leone_add_layernorm(float* x, const float* delta, const void* dw,
     const AnyVec vdw{dw, w_dtype}, vdb{db, w_dtype}, vw{w, w_dtype}, vb{b, w_dtype};
     const int stage_delta = (delta && static_cast<size_t>(hidden) * 2 * sizeof(float) <= 64 * 1024) ? 1 : 0;
     const size_t shared = static_cast<size_t>(hidden) * sizeof(float) * (stage_delta ? 2 : 1);
-    if (y_dtype == kF32)
-        add_layernorm_kernel<float><<<n_out, kNormThreads, shared, stream>>>(x, delta, vdw, vdb, deps, vw, vb, eps,
-                                                                            static_cast<float*>(y), rows, hidden, vconv, taps,
-                                                                            conv_state, write_state, positions, row_entry, entry_slots, stage_delta);
-    else
-        add_layernorm_kernel<bf16_t><<<n_out, kNormThreads, shared, stream>>>(x, delta, vdw, vdb, deps, vw, vb, eps,
-                                                                             static_cast<bf16_t*>(y), rows, hidden, vconv, taps,
-                                                                             conv_state, write_state, positions, row_entry, entry_slots, stage_delta);
+#define LEONE_LAYERNORM(T, THREADS)                                                                                        \
+    add_layernorm_kernel<T, THREADS><<<n_out, THREADS, shared, stream>>>(x, delta, vdw, vdb, deps, vw, vb, eps, static_cast<T*>(y), \
+                                                                         rows, hidden, vconv, taps, conv_state, write_state,   \
+                                                                         positions, row_entry, entry_slots, stage_delta)
+    const bool many = n_out >= kNormManyRows;
+    if (y_dtype == kF32) {
+        if (many) LEONE_LAYERNORM(float, kNormThreadsMany);
+        else LEONE_LAYERNORM(float, kNormThreadsFew);
+    } else {
+        if (many) LEONE_LAYERNORM(bf16_t, kNormThreadsMany);
+        else LEONE_LAYERNORM(bf16_t, kNormThreadsFew);
+    }
+#undef LEONE_LAYERNORM
     LEONE_LAUNCH_CHECK("add_layernorm");
     return 0;
 }
@@ -311,12 +336,13 @@ extern "C" int leone_causal_conv(const void* in, int in_dtype, long in_stride, v
     LEONE_REQUIRE(!write_state || single_rows || (spans && entries > 0 && entries <= 65535),
                   "causal_conv: the state's update needs the entries' spans");
     const AnyVec vw{w, w_dtype};
-    const dim3 grid(rows, ceil_div(channels, 256));
+    const int per_block = rows >= kNormManyRows ? kConvRows : 1;
+    const dim3 grid(ceil_div(rows, per_block), ceil_div(channels, 256));
 #define LEONE_CONV(TIN, TOUT)                                                                                         \
     causal_conv_kernel<TIN, TOUT><<<grid, 256, 0, stream>>>(static_cast<const TIN*>(in), in_stride, static_cast<TOUT*>(out), \
                                                             out_stride, vw, state, positions, row_entry, entry_slots, \
-                                                            channels, taps, add_input, act,                          \
-                                                            (write_state && single_rows) ? state : nullptr)
+                                                            rows, channels, taps, add_input, act,                    \
+                                                            (write_state && single_rows) ? state : nullptr, per_block)
     if (in_dtype == kF32 && out_dtype == kF32) LEONE_CONV(float, float);
     else if (in_dtype == kF32) LEONE_CONV(float, bf16_t);
     else if (out_dtype == kF32) LEONE_CONV(bf16_t, float);
@@ -367,7 +393,8 @@ extern "C" int leone_rms_mix(const float* const* branch_rows, const void* const*
         in.rows[b] = branch_rows[b];
         in.gain[b] = AnyVec{gains[b], gain_dtype};
     }
-    rms_mix_kernel<<<rows, kNormThreads, 0, stream>>>(in, branches, eps, scale, out, hidden);
+    if (rows >= kNormManyRows) rms_mix_kernel<kNormThreadsMany><<<rows, kNormThreadsMany, 0, stream>>>(in, branches, eps, scale, out, hidden);
+    else rms_mix_kernel<kNormThreadsFew><<<rows, kNormThreadsFew, 0, stream>>>(in, branches, eps, scale, out, hidden);
     LEONE_LAUNCH_CHECK("rms_mix");
     return 0;
 }
