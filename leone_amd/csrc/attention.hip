@@ -20,7 +20,7 @@ namespace leone {
 
 constexpr int kRowThreads = 256;
 constexpr int kRowWaves = kRowThreads / kWave;
-constexpr int kRowDimsPerLane = 8;                      // keys and values of up to 512 elements a head
+constexpr int kRowDimsPerLane = 4;                      // keys and values of up to 256 elements a head
 constexpr int kRowMaxHeadDim = kWave * kRowDimsPerLane;
 
 // One block per (row, query head).  Wave w takes keys first + w, first + w + 4,
