@@ -48,7 +48,7 @@ SMALL = {
                             mlstm(2, 72, 70, 10.0)]),
     "S": config(48, 130, 4, [mlstm(2, 16, 16, 12.0), delta(2, 2, 16, 16, 4)]),          # no paged cache at all
     # keys and values of one size, a multiple of 64: in bfloat16 the attention branch goes to the matrix-core kernels
-    "T": config(128, 257, 3, [parallel(4, 2, 64, 64, 32, 2, 32, 64, 32, [0.96, 0.999], ff=160), mlstm(2, 32, 64, 9.0),
+    "T": config(128, 257, 3, [parallel(4, 2, 64, 64, 32, 2, 32, 64, 32, [0.96, 0.999], ff=160), mlstm(2, 48, 80, 9.0),
                               parallel(2, 1, 128, 128, 128, 1, 64, 32, 16, [0.9])]),
 }
 RANKS = {"P": (8, 16), "Q": (12, 8), "R": (5, 8), "S": (8, 8), "T": (8, 8)}      # (a_rank, g_rank); 12 and 5: inner sizes off the runs of 8

@@ -42,10 +42,6 @@ def input_convolution(h, w):
     return h + causal_taps(h, w)
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def rotate_half(x, positions, dims, base):
     """x [steps, heads, size]: the first ``dims`` elements of every head turn in pairs (i, i + dims/2) by the
     angle position * base^(-2i/dims); the rest is left alone."""
