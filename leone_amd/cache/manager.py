@@ -56,10 +56,15 @@ class CacheError(RuntimeError):
 
 @dataclass(frozen=True)
 class GroupSpec:
-    """Pages of one group: ``window`` None keeps every position, else only the last ``window``."""
+    """Pages of one group: ``window`` None keeps every position, else only the last ``window`` and, whatever the
+    window, the first ``keep_first`` (the pages that hold them are never handed back by a window that passes)."""
     num_pages: int
     page_tokens: int
     window: Optional[int] = None
+    keep_first: int = 0
+
+    def kept_blocks(self) -> int:
+        return 0 if self.window is None else -(-self.keep_first // self.page_tokens)
 
 
 class RequestKeys:
@@ -116,7 +121,7 @@ class CacheManager:
         if max_requests <= 0 or max_context <= 0:
             raise ValueError("max_requests and max_context must be positive")
         for g in groups:
-            if g.num_pages <= 0 or g.page_tokens <= 0 or (g.window is not None and g.window <= 0):
+            if g.num_pages <= 0 or g.page_tokens <= 0 or (g.window is not None and g.window <= 0) or g.keep_first < 0:
                 raise ValueError(f"invalid cache group {g}")
         self.groups = list(groups)
         self.max_requests = max_requests
@@ -129,6 +134,9 @@ class CacheManager:
         self.handle = self._lib.leone_cache_create(flat, len(groups), max_requests, max_context)
         if not self.handle:
             raise ValueError(hostlib.last_error())
+        for i, g in enumerate(groups):
+            if g.window is not None and g.keep_first:
+                self._checked(self._lib.leone_cache_set_keep_first(self.handle, i, g.keep_first))
         self._max_blocks = [self._lib.leone_cache_max_blocks(self.handle, g) for g in range(len(groups))]
         self._table_buffers = [(c_int * max(1, width))() for width in self._max_blocks]
 
@@ -303,7 +311,9 @@ class CacheManager:
                 total = length + self._checked(self._lib.leone_cache_pending(self.handle, self._key(request)))
                 first = 0 if g.window is None else max(0, length - (g.window - 1)) // g.page_tokens
                 if total:
-                    for b in range(first, (total - 1) // g.page_tokens + 1):
+                    for b in range(0, (total - 1) // g.page_tokens + 1):
+                        if b < first and b >= g.kept_blocks():
+                            continue
                         if b >= len(table) or table[b] < 0:
                             raise CacheError(f"group {gi}: {request!r} has no page for block {b}")
             for page in range(g.num_pages):

@@ -43,7 +43,7 @@ class DevicePools:
         for gi, need in enumerate(self.group_needs):
             pages = num_pages[gi] if isinstance(num_pages, dict) else num_pages
             self.group_specs.append(GroupSpec(pages, getattr(need, "page_tokens", None) or page_tokens,
-                                              getattr(need, "window", None)))
+                                              getattr(need, "window", None), int(getattr(need, "keep_first", 0) or 0)))
         for slot, gi in self.group_of_slot.items():
             spec = self.group_specs[gi]
             self.paged[slot] = needs[slot].allocate(spec.num_pages, spec.page_tokens, dtype, self.device)

@@ -2,7 +2,8 @@
 //
 // For a query row at absolute position `pos` of its request and query head h,
 // with kv head h / (q_heads / kv_heads): scores s_j = (q . K[j]) * scale for
-// keys j in [first, pos], first = 0 or pos - window + 1 for a windowed layer;
+// keys j in [first, pos], first = 0 or pos - window + 1 for a windowed layer, and, if the layer keeps its
+// first tokens in sight, also for the keys j < keep_first (at their own places in the cache);
 // softmax over them; out = sum_j p_j V[j].  This is the reference's recurrence
 // (crates/leone/src/cpu.rs:2299-2421: scale after the dot, running maximum,
 // rescaled sum and accumulator), with the keys found through the request's block
@@ -32,7 +33,7 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
                                       const int* __restrict__ positions, const int* __restrict__ row_entry,
                                       const int* __restrict__ block_table, int max_blocks, int q_heads,
                                       int kv_heads, int head_dim, int v_dim, int page_tokens, float scale, int window,
-                                      const float* __restrict__ gate, long gate_stride) {
+                                      const float* __restrict__ gate, long gate_stride, int keep_first, int gate_each) {
     __shared__ float sm_m[kRowWaves];
     __shared__ float sm_l[kRowWaves];
     __shared__ float sm_acc[kRowWaves][kRowMaxHeadDim];
@@ -58,7 +59,11 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
     float acc[kRowDimsPerLane];
 #pragma unroll
     for (int i = 0; i < kRowDimsPerLane; ++i) acc[i] = 0.f;
-    for (int j = first + wave; j <= pos; j += kRowWaves) {
+    // the kept first keys that the window has left behind come first, then the window's
+    const int kept = keep_first < first ? keep_first : first;
+    const int reach = kept + pos - first + 1;
+    for (int t = wave; t < reach; t += kRowWaves) {
+        const int j = t < kept ? t : first + (t - kept);
         const int page = table[j / page_tokens];
         if (page < 0) {  // an unmapped block: poison the result instead of reading outside the pool
             l = __builtin_nanf("");
@@ -93,9 +98,12 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
     __syncthreads();
 
     T* orow = out + (static_cast<long>(row) * q_heads + head) * v_dim;
-    // an output gate of the head: the result times sigmoid(gate[row, head])
-    const float open = gate ? 1.0f / (1.0f + expf(-gate[static_cast<long>(row) * gate_stride + head])) : 1.0f;
+    // an output gate: the result times sigmoid(gate[row, head]), or, with a gate for each element, times
+    // sigmoid(gate[row, head * v_dim + d])
+    const float* gate_row = gate ? gate + static_cast<long>(row) * gate_stride + (gate_each ? static_cast<long>(head) * v_dim : head) : nullptr;
+    const float open_head = (gate && !gate_each) ? 1.0f / (1.0f + expf(-gate_row[0])) : 1.0f;
     for (int d = threadIdx.x; d < v_dim; d += kRowThreads) {
+        const float open = (gate && gate_each) ? 1.0f / (1.0f + expf(-gate_row[d])) : open_head;
         float top = sm_m[0];
 #pragma unroll
         for (int w = 1; w < kRowWaves; ++w) top = fmaxf(top, sm_m[w]);
@@ -120,6 +128,17 @@ extern "C" int leone_attention_rows(const void* q, void* out, const void* k_pool
                                     int max_blocks, int rows, int q_heads, int kv_heads, int head_dim, int v_dim,
                                     int page_tokens, float scale, int window, const float* gate, long gate_stride,
                                     hipStream_t stream) {
+    return leone_attention_rows_kept(q, out, k_pool, v_pool, dtype, positions, row_entry, block_table, max_blocks, rows,
+                                     q_heads, kv_heads, head_dim, v_dim, page_tokens, scale, window, gate, gate_stride, 0, 0, stream);
+}
+
+// keep_first: keys at positions below it stay in sight of a windowed layer.  gate_each: the gate holds a value
+// for every element of every head ([rows, q_heads * v_dim] within rows of gate_stride) instead of one a head.
+extern "C" int leone_attention_rows_kept(const void* q, void* out, const void* k_pool, const void* v_pool, int dtype,
+                                         const int* positions, const int* row_entry, const int* block_table,
+                                         int max_blocks, int rows, int q_heads, int kv_heads, int head_dim, int v_dim,
+                                         int page_tokens, float scale, int window, const float* gate, long gate_stride,
+                                         int keep_first, int gate_each, hipStream_t stream) {
     LEONE_REQUIRE(dtype == kF32 || dtype == kBF16, "attention_rows: unknown element type %d", dtype);
     LEONE_REQUIRE(q && out && k_pool && v_pool && positions && row_entry && block_table, "attention_rows: null pointer");
     LEONE_REQUIRE(rows > 0 && q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
@@ -127,7 +146,9 @@ extern "C" int leone_attention_rows(const void* q, void* out, const void* k_pool
     LEONE_REQUIRE(q_heads <= 65535, "attention_rows: at most 65535 query heads");
     LEONE_REQUIRE(head_dim > 0 && head_dim <= kRowMaxHeadDim, "attention_rows: head_dim %d must be in 1..%d", head_dim, kRowMaxHeadDim);
     LEONE_REQUIRE(v_dim > 0 && v_dim <= kRowMaxHeadDim, "attention_rows: value size %d must be in 1..%d", v_dim, kRowMaxHeadDim);
-    LEONE_REQUIRE(!gate || gate_stride >= q_heads, "attention_rows: gate rows of %ld for %d heads", gate_stride, q_heads);
+    LEONE_REQUIRE(!gate || gate_stride >= (gate_each ? static_cast<long>(q_heads) * v_dim : q_heads),
+                  "attention_rows: gate rows of %ld for %d heads", gate_stride, q_heads);
+    LEONE_REQUIRE(keep_first >= 0, "attention_rows: keep_first %d must not be negative", keep_first);
     LEONE_REQUIRE(page_tokens > 0 && max_blocks > 0, "attention_rows: page_tokens %d and max_blocks %d must be positive", page_tokens, max_blocks);
     LEONE_REQUIRE(head_dim % 8 == 0 && page_tokens % 8 == 0,
                   "attention_rows: head_dim %d and page_tokens %d must be multiples of 8", head_dim, page_tokens);
@@ -137,12 +158,12 @@ extern "C" int leone_attention_rows(const void* q, void* out, const void* k_pool
         attention_rows_kernel<float><<<grid, kRowThreads, 0, stream>>>(
             static_cast<const float*>(q), static_cast<float*>(out), static_cast<const float*>(k_pool),
             static_cast<const float*>(v_pool), positions, row_entry, block_table, max_blocks, q_heads, kv_heads,
-            head_dim, v_dim, page_tokens, scale, window, gate, gate_stride);
+            head_dim, v_dim, page_tokens, scale, window, gate, gate_stride, keep_first, gate_each);
     else
         attention_rows_kernel<bf16_t><<<grid, kRowThreads, 0, stream>>>(
             static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_pool),
             static_cast<const bf16_t*>(v_pool), positions, row_entry, block_table, max_blocks, q_heads, kv_heads,
-            head_dim, v_dim, page_tokens, scale, window, gate, gate_stride);
+            head_dim, v_dim, page_tokens, scale, window, gate, gate_stride, keep_first, gate_each);
     LEONE_LAUNCH_CHECK("attention_rows");
     return 0;
 }

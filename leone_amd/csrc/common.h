@@ -161,4 +161,12 @@ void set_error(const char* fmt, ...);
 
 inline int ceil_div(long a, long b) { return static_cast<int>((a + b - 1) / b); }
 
+// The activation of the gate of a gated feed-forward: 0 silu(g) = g / (1 + exp(-g)); 1 the tanh form of gelu,
+// 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))).
+enum GateAct : int { kGateSilu = 0, kGateGeluTanh = 1 };
+__device__ inline float gate_act(float g, int act) {
+    if (act == kGateGeluTanh) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.0f + expf(-g));
+}
+
 }  // namespace leone

@@ -53,6 +53,7 @@ struct FusedArgs {
     float* squares_out;        // prepare: [M, ceil(N / 16)]
     const void* next_gain;     // prepare: [N]
     int next_gain_dtype;
+    int act;                   // gated: the gate's activation (GateAct)
 };
 
 __device__ inline bf16x8 fz8() {
@@ -243,7 +244,7 @@ gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float gate = sum[r];
-                out[r] = from_float<bf16_t>((gate / (1.0f + expf(-gate))) * up[r]);
+                out[r] = from_float<bf16_t>(gate_act(gate, a.act) * up[r]);
             }
         }
         return;
@@ -327,6 +328,7 @@ using namespace leone;
 // in_mode: 0 plain (x bfloat16 [m,k]), 1 norm (x float32 stream, optional rows, gain, eps), 2 prepared (x bfloat16
 // [m,k] and squares_in float32 [m, ceil(k / 16)] as an earlier call's out_mode 3 wrote them, eps).
 // out_mode: 0 store (y of out_dtype [m,n]), 1 residual (y float32 [m,n] += product), 2 gated (y bfloat16 [m,n/2]),
+// 4 gated with the tanh form of gelu on the gate instead of silu,
 // 3 prepare (as 1, and operand_out bfloat16 [m,n] = bf16(y * next_gain), squares_out float32 [m, ceil(n / 16)]).
 extern "C" int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const void* gain, int gain_dtype,
                                      float eps, const void* w, int w_tiled, void* y, int out_mode, int out_dtype, int m, int n,
@@ -346,14 +348,16 @@ extern "C" int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows
     LEONE_REQUIRE(in_mode != kInPrepared || (k % 64 == 0 && static_cast<long>(m) * (k / 64) <= 8 * 256 &&
                                              reinterpret_cast<uintptr_t>(squares_in) % 16 == 0),
                   "gemm_fused: the prepared input takes K %d a multiple of 64 with rows x K / 64 up to 2048", k);
-    LEONE_REQUIRE(out_mode >= kOutStore && out_mode <= kOutPrepare, "gemm_fused: unknown output mode %d", out_mode);
+    LEONE_REQUIRE(out_mode >= kOutStore && out_mode <= kOutPrepare + 1, "gemm_fused: unknown output mode %d", out_mode);
+    const int act = out_mode == kOutPrepare + 1 ? kGateGeluTanh : kGateSilu;
+    if (out_mode == kOutPrepare + 1) out_mode = kOutGated;
     LEONE_REQUIRE(out_mode != kOutGated || n % 16 == 0, "gemm_fused: gated output needs N %d to be a multiple of 16", n);
     LEONE_REQUIRE(out_mode != kOutStore || out_dtype == kF32 || out_dtype == kBF16, "gemm_fused: unknown output type");
     LEONE_REQUIRE(out_mode != kOutPrepare || (operand_out && squares_out && next_gain &&
                                               (next_gain_dtype == kF32 || next_gain_dtype == kBF16)),
                   "gemm_fused: the prepare output needs room for the operand and the sums, and the next gain");
     FusedArgs a{x, rows, gain, gain_dtype, eps, static_cast<const bf16_t*>(w), y, m, n, k,
-                squares_in, static_cast<bf16_t*>(operand_out), squares_out, next_gain, next_gain_dtype};
+                squares_in, static_cast<bf16_t*>(operand_out), squares_out, next_gain, next_gain_dtype, act};
 #define LEONE_FUSED_OUT(IN)                                                                  \
     switch (out_mode) {                                                                      \
         case kOutStore:                                                                      \

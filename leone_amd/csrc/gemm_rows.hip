@@ -48,6 +48,7 @@ struct RowsArgs {
     long plane;        // elements between two planes of y (kRowsPlanes)
     int m, n, k;
     int chunks_per_split;
+    int act;           // gated: the gate's activation (GateAct)
 };
 
 
@@ -250,7 +251,7 @@ gemm_rows_kernel(RowsArgs a) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const float gate = acc[t][r];
-                    v[r] = (gate / (1.0f + expf(-gate))) * up[r];
+                    v[r] = gate_act(gate, a.act) * up[r];
                 }
                 uint2 packed;
                 packed.x = bf16_bits_from_float(v[0]) | (static_cast<uint32_t>(bf16_bits_from_float(v[1])) << 16);
@@ -377,7 +378,9 @@ extern "C" int leone_gemm_rows_bf16(const void* x, const void* w, int w_tiled, v
                   "gemm_rows: tiled weights need K %d to be a multiple of 64", k);
     LEONE_REQUIRE(m > 0 && m <= 128, "gemm_rows: rows %d must be in 1..128", m);
     LEONE_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_rows: sizes %d x %d: K must be a positive multiple of 8", n, k);
-    LEONE_REQUIRE(out_mode >= kRowsStore && out_mode <= kRowsPlanes, "gemm_rows: unknown output mode %d", out_mode);
+    LEONE_REQUIRE(out_mode >= kRowsStore && out_mode <= kRowsPlanes + 1, "gemm_rows: unknown output mode %d", out_mode);
+    const int act = out_mode == kRowsPlanes + 1 ? kGateGeluTanh : kGateSilu;     // 4: as 2 with the tanh form of gelu on the gate
+    if (out_mode == kRowsPlanes + 1) out_mode = kRowsGated;
     LEONE_REQUIRE(out_mode != kRowsGated || n % 16 == 0, "gemm_rows: gated output needs N %d to be a multiple of 16", n);
     LEONE_REQUIRE(out_mode != kRowsStore || out_dtype == kF32 || out_dtype == kBF16, "gemm_rows: unknown output type");
     LEONE_REQUIRE(waves == 4 || waves == 6 || waves == 8, "gemm_rows: %d tiles of W a workgroup", waves);
@@ -390,7 +393,7 @@ extern "C" int leone_gemm_rows_bf16(const void* x, const void* w, int w_tiled, v
     const int per = ceil_div(chunks, splits);
     LEONE_REQUIRE(per * (splits - 1) < chunks, "gemm_rows: %d ranges of K would leave one empty (%d chunks)", splits, chunks);
     LEONE_REQUIRE(out_mode != kRowsPlanes || plane >= static_cast<long>(m) * n, "gemm_rows: planes overlap");
-    RowsArgs a{static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, plane, m, n, k, per};
+    RowsArgs a{static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, plane, m, n, k, per, act};
     int status = 0;
 #define LEONE_ROWS_CASE(MT) \
     case MT: status = launch_rows_waves<MT>(a, out_mode, out_dtype, splits, waves, ways, w_tiled != 0, stream); break;

@@ -81,6 +81,9 @@ void* leone_cache_create(const int* groups, int n_groups, int max_requests, int 
     });
     return made;
 }
+int leone_cache_set_keep_first(void* cache, int group, int positions) {
+    return guarded([&]() -> long { cache_of(cache).set_keep_first(group, positions); return 0; });
+}
 void leone_cache_destroy(void* cache) { delete static_cast<CacheManager*>(cache); }
 
 int leone_cache_admit(void* cache, int64_t request) {

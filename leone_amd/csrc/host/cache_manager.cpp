@@ -32,6 +32,13 @@ CacheManager::CacheManager(std::vector<GroupSpec> groups, int max_requests, int 
     for (int i = 0; i < max_requests; ++i) free_slots_[i] = max_requests - 1 - i;
 }
 
+void CacheManager::set_keep_first(int g, int positions) {
+    if (g < 0 || g >= group_count()) throw CacheError("no cache group " + std::to_string(g));
+    if (positions < 0) throw std::invalid_argument("keep_first must not be negative");
+    if (!requests_.empty()) throw CacheError("keep_first is set before requests are admitted");
+    groups_[g].keep_first = positions;
+}
+
 int CacheManager::max_blocks(int g) const {
     const int pt = groups_.at(g).page_tokens;
     return (max_context_ + pt - 1) / pt;
@@ -147,7 +154,8 @@ int CacheManager::fork(RequestKey parent, RequestKey child, int tokens) {
         const int first = g.window == 0 ? 0 : std::max(0, shared - (g.window - 1)) / g.page_tokens;
         const std::vector<int>& table = source.tables[gi];
         std::vector<int> pages(blocks, -1);
-        for (int b = first; b < blocks; ++b) {
+        for (int b = 0; b < blocks; ++b) {
+            if (b < first && b >= g.kept_blocks()) continue;       // behind the window and not among the kept first
             if (b >= static_cast<int>(table.size()) || table[b] < 0)
                 throw CacheError("group " + std::to_string(gi) + ": the parent's window has passed block " +
                                  std::to_string(b) + "; fork later tokens");
@@ -182,8 +190,8 @@ void CacheManager::truncate(RequestKey request, int position) {
                              " is shared; truncate to a multiple of " + std::to_string(g.page_tokens));
         if (g.window != 0) {
             const int reach = std::max(0, position - (g.window - 1)) / g.page_tokens;
-            for (int b = reach; b < std::min(keep, size); ++b)
-                if (table[b] < 0)
+            for (int b = 0; b < std::min(keep, size); ++b)
+                if ((b >= reach || b < g.kept_blocks()) && table[b] < 0)
                     throw CacheError("group " + std::to_string(gi) + ": keys before position " + std::to_string(position) +
                                      " have left the window; they cannot be brought back by truncation");
         }
@@ -242,7 +250,7 @@ void CacheManager::commit(RequestKey request, int tokens) {
         const int reach = state.length - (g.window - 1);
         std::vector<int>& table = state.tables[gi];
         const int end = std::min(static_cast<int>(table.size()), std::max(0, reach) / g.page_tokens);
-        for (int b = 0; b < end; ++b)
+        for (int b = g.kept_blocks(); b < end; ++b)               // the kept first positions keep their pages
             if (table[b] >= 0) {
                 drop(gi, table[b]);
                 table[b] = -1;

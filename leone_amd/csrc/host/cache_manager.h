@@ -34,6 +34,10 @@ struct GroupSpec {
     int num_pages;
     int page_tokens;
     int window;   // 0: every position is kept; otherwise only the last `window`
+    int keep_first = 0;   // of a windowed group: the first positions stay in sight whatever the window, so their pages stay
+
+    // Pages that hold the kept first positions (they are never handed back by a window that passes).
+    int kept_blocks() const { return window == 0 ? 0 : (keep_first + page_tokens - 1) / page_tokens; }
 };
 
 // A reservation needs more free pages than a group has; nothing was changed.
@@ -62,6 +66,8 @@ public:
     int max_requests() const { return max_requests_; }
     int max_context() const { return max_context_; }
     int max_blocks(int g) const;
+    // The first `positions` positions of group g stay readable whatever its window (before any request is admitted).
+    void set_keep_first(int g, int positions);
     bool has(RequestKey request) const { return requests_.count(request) != 0; }
     std::vector<RequestKey> requests() const;   // every admitted request, ascending
     int length(RequestKey request) const { return get(request).length; }

@@ -23,6 +23,8 @@ const char* leone_host_last_error(void);
 
 // ---- cache manager.  groups: n_groups x (num_pages, page_tokens, window or 0).
 void* leone_cache_create(const int* groups, int n_groups, int max_requests, int max_context);
+// Of a windowed group: its first `positions` positions stay readable whatever the window (their pages are kept).
+int leone_cache_set_keep_first(void* cache, int group, int positions);
 void leone_cache_destroy(void* cache);
 int leone_cache_admit(void* cache, int64_t request);                                  // the state slot
 int leone_cache_fork(void* cache, int64_t parent, int64_t child, int tokens);         // tokens the child holds

@@ -62,7 +62,8 @@ Reject Scheduler::reject_reason(RequestKey request, int prompt, std::int64_t out
         } else {
             const std::int64_t portion = std::min(policy_.prefill_chunk_tokens, policy_.max_step_tokens);
             const std::int64_t span = std::min<std::int64_t>(held, g.window - 1 + portion);
-            need = (span + g.page_tokens - 1) / g.page_tokens + 1;
+            need = std::min<std::int64_t>((span + g.page_tokens - 1) / g.page_tokens + 1 + g.kept_blocks(),
+                                          (held + g.page_tokens - 1) / g.page_tokens);
         }
         if (need > g.num_pages) return Reject::KvCapacity;
     }
@@ -266,7 +267,9 @@ bool Scheduler::room_for(int tokens) const {
         const GroupSpec& g = cache_.group(gi);
         const std::int64_t span =
             g.window == 0 ? tokens : std::min<std::int64_t>(tokens, g.window - 1 + policy_.prefill_chunk_tokens);
-        if ((span + g.page_tokens - 1) / g.page_tokens > cache_.free_pages(gi)) return false;
+        const std::int64_t pages = std::min<std::int64_t>((span + g.page_tokens - 1) / g.page_tokens + g.kept_blocks(),
+                                                          (tokens + g.page_tokens - 1) / g.page_tokens);
+        if (pages > cache_.free_pages(gi)) return false;
     }
     return true;
 }

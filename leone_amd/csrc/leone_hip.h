@@ -253,4 +253,38 @@ int leone_delta_scan(const float* qkv, long stride, int q_off, int k_off, int v_
                      hipStream_t stream);
 int leone_delta_chain(const int* links, int n_links, float* work, long work_stride, const float* transition, float* state,
                       long slot_stride, int heads, int dim, int vdim, int write_state, hipStream_t stream);
+
+// ---- a token table with a learned position table added, norms behind sublayers, kept first keys, routed experts ----
+// leone_embed, and place_table[positions[r], :] (of the table's type, [places, hidden]) added unscaled.
+int leone_embed_placed(const void* table, int dtype, const int* tokens, float* out, int rows, int hidden, int vocab,
+                       float scale, const void* place_table, const int* positions, int places, hipStream_t stream);
+// gate_up as for leone_swiglu; act: 0 silu, 1 the tanh form of gelu on the gate.
+int leone_glu(const void* gate_up, void* out, int dtype, int rows, int ffn, int act, hipStream_t stream);
+// x[r] += rmsnorm(sum of the delta's planes)[r] * gain (delta float32, may be null); then y[r] = x[r] in y_dtype
+// (y may be null), or, with gain2, y[i] = rmsnorm(x[rows ? rows[i] : i]) * gain2 (with rows, x is not written).
+int leone_add_normed(float* x, const float* delta, int delta_planes, long delta_plane, const void* gain, int gain_dtype,
+                     float eps, void* y, int y_dtype, const void* gain2, int gain2_dtype, float eps2, const int* rows,
+                     int n_rows, int hidden, hipStream_t stream);
+// leone_attention_rows with the keys below keep_first kept in sight of a windowed layer, and with gate_each a
+// gate value for every element of every head ([rows, q_heads * v_dim] within rows of gate_stride).
+int leone_attention_rows_kept(const void* q, void* out, const void* k_pool, const void* v_pool, int dtype,
+                              const int* positions, const int* row_entry, const int* block_table, int max_blocks,
+                              int rows, int q_heads, int kv_heads, int head_dim, int v_dim, int page_tokens,
+                              float scale, int window, const float* gate, long gate_stride, int keep_first,
+                              int gate_each, hipStream_t stream);
+// Router: chosen int32 [rows, top], weight float32 [rows, top] from logits float32 [rows, total] (see routed.hip).
+int leone_route_max_outputs();
+int leone_route_topk(const float* logits, const void* correction, int correction_dtype, int* chosen, float* weight,
+                     int rows, int total, int top, int group_count, int group_keep, hipStream_t stream);
+// Pairs (row, place) of the experts below `experts` gathered in tiles of leone_moe_tile_pairs() pairs of one expert:
+// tile_expert int32 [max_tiles] (-1: unused), tile_pairs int32 [max_tiles, tile pairs] (-1: empty);
+// max_tiles >= min(pairs, pairs / tile pairs + experts).
+int leone_moe_tile_pairs();
+int leone_moe_plan(const int* chosen, int pairs, int experts, int* tile_expert, int* tile_pairs, int max_tiles,
+                   hipStream_t stream);
+int leone_moe_product(const void* x, const void* w, void* y, const float* pair_weight, int dtype, int gated,
+                      const int* tile_expert, const int* tile_pairs, int max_tiles, int top, int n, int k, int act,
+                      hipStream_t stream);
+int leone_moe_combine(const float* pair_out, const int* chosen, const float* weight, const void* x, int dtype,
+                      const float* extra, float* out, int rows, int top, int experts, int hidden, hipStream_t stream);
 }

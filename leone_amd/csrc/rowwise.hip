@@ -17,7 +17,8 @@ namespace leone {
 // ---- embedding -------------------------------------------------------------
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
-                             float* __restrict__ out, int hidden, int vocab, float scale) {
+                             float* __restrict__ out, int hidden, int vocab, float scale,
+                             const T* __restrict__ place_table, const int* __restrict__ positions, int places) {
     const int row = blockIdx.x;
     const int token = tokens[row];
     float* dst = out + static_cast<long>(row) * hidden;
@@ -27,6 +28,13 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
         return;
     }
     const T* src = table + static_cast<long>(token) * hidden;
+    if (place_table != nullptr) {
+        // a learned vector of the row's position is added (not scaled); the host checks the bound
+        const int pos = positions[row];
+        const T* at = place_table + static_cast<long>(pos < places ? (pos < 0 ? 0 : pos) : places - 1) * hidden;
+        for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = to_float(src[c]) * scale + to_float(at[c]);
+        return;
+    }
     for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = to_float(src[c]) * scale;
 }
 
@@ -184,7 +192,7 @@ struct alignas(8 * sizeof(T)) Run8 {
 };
 template <typename T>
 __global__ void __launch_bounds__(256)
-swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long rows, int ffn) {
+swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long rows, int ffn, int act) {
     const int groups = ffn / 8;
     const int group = blockIdx.x * blockDim.x + threadIdx.x;
     if (group >= groups) return;
@@ -196,7 +204,7 @@ swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long rows, int
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const float g = to_float(gate.v[i]);
-            y.v[i] = from_float<T>((g / (1.0f + expf(-g))) * to_float(up.v[i]));
+            y.v[i] = from_float<T>(gate_act(g, act) * to_float(up.v[i]));
         }
         *reinterpret_cast<Run8<T>*>(out + r * ffn + 8 * static_cast<long>(group)) = y;
     }
@@ -598,18 +606,27 @@ extern "C" int leone_soft_cap(float* x, long n, float cap, hipStream_t stream) {
     return 0;
 }
 
-extern "C" int leone_embed(const void* table, int dtype, const int* tokens, float* out, int rows,
-                           int hidden, int vocab, float scale, hipStream_t stream) {
+extern "C" int leone_embed_placed(const void* table, int dtype, const int* tokens, float* out, int rows,
+                                  int hidden, int vocab, float scale, const void* place_table, const int* positions,
+                                  int places, hipStream_t stream) {
     if (check_dtype(dtype, "embed")) return 1;
     LEONE_REQUIRE(table && tokens && out, "embed: null pointer");
+    LEONE_REQUIRE(!place_table || (positions && places > 0), "embed: a position table needs the rows' positions");
     LEONE_REQUIRE(rows > 0 && hidden > 0 && vocab > 0, "embed: rows %d hidden %d vocab %d must be positive", rows, hidden, vocab);
     const int threads = hidden >= 1024 ? 256 : 64;
     if (dtype == kF32)
-        embed_kernel<float><<<rows, threads, 0, stream>>>(static_cast<const float*>(table), tokens, out, hidden, vocab, scale);
+        embed_kernel<float><<<rows, threads, 0, stream>>>(static_cast<const float*>(table), tokens, out, hidden, vocab, scale,
+                                                          static_cast<const float*>(place_table), positions, places);
     else
-        embed_kernel<bf16_t><<<rows, threads, 0, stream>>>(static_cast<const bf16_t*>(table), tokens, out, hidden, vocab, scale);
+        embed_kernel<bf16_t><<<rows, threads, 0, stream>>>(static_cast<const bf16_t*>(table), tokens, out, hidden, vocab, scale,
+                                                           static_cast<const bf16_t*>(place_table), positions, places);
     LEONE_LAUNCH_CHECK("embed");
     return 0;
+}
+
+extern "C" int leone_embed(const void* table, int dtype, const int* tokens, float* out, int rows,
+                           int hidden, int vocab, float scale, hipStream_t stream) {
+    return leone_embed_placed(table, dtype, tokens, out, rows, hidden, vocab, scale, nullptr, nullptr, 0, stream);
 }
 
 template <typename TD, typename TG, typename TY>
@@ -670,8 +687,10 @@ extern "C" int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, i
     return 0;
 }
 
-extern "C" int leone_swiglu(const void* gate_up, void* out, int dtype, int rows, int ffn, hipStream_t stream) {
+// act: the gate's activation (GateAct: 0 silu, 1 the tanh form of gelu).
+extern "C" int leone_glu(const void* gate_up, void* out, int dtype, int rows, int ffn, int act, hipStream_t stream) {
     if (check_dtype(dtype, "swiglu")) return 1;
+    LEONE_REQUIRE(act == kGateSilu || act == kGateGeluTanh, "glu: unknown activation %d", act);
     LEONE_REQUIRE(gate_up && out, "swiglu: null pointer");
     LEONE_REQUIRE(rows > 0 && ffn > 0 && ffn % 8 == 0, "swiglu: rows %d, width %d: the width must be a positive multiple of 8", rows, ffn);
     const uintptr_t run = 8 * (dtype == kF32 ? sizeof(float) : sizeof(bf16_t));
@@ -679,11 +698,15 @@ extern "C" int leone_swiglu(const void* gate_up, void* out, int dtype, int rows,
                   "swiglu: input and output must be aligned to %d bytes", static_cast<int>(run));
     const dim3 grid(ceil_div(ffn / 8, 256), rows < 32768 ? rows : 32768);
     if (dtype == kF32)
-        swiglu_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(gate_up), static_cast<float*>(out), rows, ffn);
+        swiglu_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(gate_up), static_cast<float*>(out), rows, ffn, act);
     else
-        swiglu_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out), rows, ffn);
+        swiglu_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out), rows, ffn, act);
     LEONE_LAUNCH_CHECK("swiglu");
     return 0;
+}
+
+extern "C" int leone_swiglu(const void* gate_up, void* out, int dtype, int rows, int ffn, hipStream_t stream) {
+    return leone_glu(gate_up, out, dtype, rows, ffn, kGateSilu, stream);
 }
 
 extern "C" int leone_rope_table(float* cos_out, float* sin_out, double theta, int rotary_dim,
@@ -712,7 +735,9 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_
     if (v_dim <= 0) v_dim = head_dim;
     const long heads_width = static_cast<long>(q_heads + kv_heads) * head_dim + static_cast<long>(kv_heads) * v_dim;
     if (row_width <= 0) row_width = heads_width;
-    LEONE_REQUIRE(row_width >= heads_width, "qk_norm_rope_write: rows of %ld elements do not hold the heads (%ld)", row_width, heads_width);
+    // a layer that reads another layer's cache may bring rows without key and value heads
+    const long needed_width = write_cache ? heads_width : static_cast<long>(q_heads) * head_dim;
+    LEONE_REQUIRE(row_width >= needed_width, "qk_norm_rope_write: rows of %ld elements do not hold the heads (%ld)", row_width, needed_width);
     LEONE_REQUIRE(v_dim % 2 == 0 && v_dim <= 2 * kWave * kMaxPairsPerLane, "qk_norm_rope_write: value size %d must be even and at most %d",
                   v_dim, 2 * kWave * kMaxPairsPerLane);
     LEONE_REQUIRE(qkv_planes == 1 || row_width == heads_width, "qk_norm_rope_write: planes come without further columns");

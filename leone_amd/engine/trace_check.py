@@ -31,6 +31,7 @@ class PoolFigures:
     num_pages: int
     page_tokens: int
     window: int = 0
+    keep_first: int = 0                      # of a windowed group: positions whose pages a passing window leaves alone
 
     def first_page(self, held: int) -> int:
         """The first page a request still holds once ``held`` positions are committed: the next row sits
@@ -43,7 +44,9 @@ class PoolFigures:
         kept after its last step, and every page up to the new end."""
         if after <= 0:
             return 0
-        return (after - 1) // self.page_tokens - self.first_page(before) + 1
+        first = self.first_page(before)
+        kept = 0 if self.window == 0 else min(first, -(-self.keep_first // self.page_tokens))
+        return (after - 1) // self.page_tokens - first + 1 + kept
 
 
 @dataclass
@@ -254,6 +257,7 @@ def verify_events(events: Iterable[tuple], figures: RunFigures) -> TraceReport:
 def figures_of(scheduler) -> RunFigures:
     """The figures of a ``Scheduler`` (its policy and its cache manager's groups)."""
     cache = scheduler.cache
-    pools = [PoolFigures(spec.num_pages, spec.page_tokens, int(spec.window or 0)) for spec in cache.groups]
+    pools = [PoolFigures(spec.num_pages, spec.page_tokens, int(spec.window or 0), int(getattr(spec, "keep_first", 0) or 0))
+             for spec in cache.groups]
     policy = scheduler.policy
     return RunFigures(pools, policy.max_live_requests, policy.max_step_tokens, policy.prefill_chunk_tokens)

@@ -25,6 +25,7 @@ PD = POINTER(c_double)
 
 _PROTOTYPES = {
     "leone_cache_create": (H, [PI, c_int, c_int, c_int]),
+    "leone_cache_set_keep_first": (c_int, [H, c_int, c_int]),
     "leone_cache_destroy": (None, [H]),
     "leone_cache_admit": (c_int, [H, c_int64]),
     "leone_cache_fork": (c_int, [H, c_int64, c_int64, c_int]),

@@ -114,12 +114,24 @@ def pack_values(v: torch.Tensor) -> torch.Tensor:
 
 
 def embed(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor] = None,
-          scale: float = 1.0) -> torch.Tensor:
-    """out[r] = table[tokens[r]] * scale as float32.  Token ids must have been checked against the table."""
+          scale: float = 1.0, position_table: Optional[torch.Tensor] = None,
+          positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[r] = table[tokens[r]] * scale as float32.  Token ids must have been checked against the table.
+    With ``position_table`` ``[places, hidden]`` (a learned vector for every position, of the table's type)
+    row r also gets position_table[positions[r]], unscaled; the caller checks positions against ``places``."""
     vocab, hidden = table.shape
     rows = tokens.numel()
     if out is None:
         out = torch.empty((rows, hidden), dtype=torch.float32, device=table.device)
+    if position_table is not None:
+        if positions is None or position_table.dtype != table.dtype or position_table.dim() != 2 or position_table.shape[1] != hidden:
+            raise KernelError(f"embed: a position table {tuple(position_table.shape)} {position_table.dtype} beside a token "
+                              f"table {tuple(table.shape)} {table.dtype} needs the rows' positions and the same type and width")
+        call("leone_embed_placed", _dev(table, "embed table"), _code(table, "embed table"),
+             _dev(tokens, "embed tokens", torch.int32, (rows,)), _dev(out, "embed out", torch.float32, (rows, hidden)),
+             rows, hidden, vocab, float(scale), _dev(position_table, "position table"),
+             _dev(positions, "positions", torch.int32, (rows,)), position_table.shape[0], _stream())
+        return out
     call("leone_embed", _dev(table, "embed table"), _code(table, "embed table"),
          _dev(tokens, "embed tokens", torch.int32, (rows,)), _dev(out, "embed out", torch.float32, (rows, hidden)),
          rows, hidden, vocab, float(scale), _stream())
@@ -159,15 +171,26 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tens
     return PreparedRows(x, gain, eps, out_dtype, out, squares, rows) if prepare else out
 
 
-def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}     # what a gated feed-forward puts on its gate
+
+
+def _gate_code(activation: str) -> int:
+    try:
+        return GATE_ACTIVATIONS[activation]
+    except KeyError:
+        raise KernelError(f"unknown gate activation {activation!r}; known: {', '.join(GATE_ACTIVATIONS)}") from None
+
+
+def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None, activation: str = "silu") -> torch.Tensor:
+    """act(gate) * up of rows that hold 8 gates, their 8 ups, and so on; ``activation`` names act."""
     rows, twice = gate_up.shape
     if twice % 2:
         raise KernelError("swiglu: input width must be even (gate columns, then up columns)")
     ffn = twice // 2
     if out is None:
         out = torch.empty((rows, ffn), dtype=gate_up.dtype, device=gate_up.device)
-    call("leone_swiglu", _dev(gate_up, "swiglu in"), _dev(out, "swiglu out", gate_up.dtype, (rows, ffn)),
-         _code(gate_up, "swiglu in"), rows, ffn, _stream())
+    call("leone_glu", _dev(gate_up, "swiglu in"), _dev(out, "swiglu out", gate_up.dtype, (rows, ffn)),
+         _code(gate_up, "swiglu in"), rows, ffn, _gate_code(activation), _stream())
     return out
 
 
@@ -210,13 +233,15 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim:
                        row_entry: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                        k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor], write_cache: bool = True,
                        out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
-                       pairing: str = "half_split", value_dim: Optional[int] = None) -> torch.Tensor:
+                       pairing: str = "half_split", value_dim: Optional[int] = None,
+                       queries_only: bool = False) -> torch.Tensor:
     """Splits the fused projection, normalises and rotates q and k heads, writes k and v into the cache.
     ``qkv`` is ``[rows, width]`` of the cache's type, or float32 (also as planes ``[p, rows, width]`` whose
     sum, in order, is meant: a product cut along K) with ``out_dtype`` naming the type of q and the cache.
     The rotation's shape comes with its tables (``_rotation_shape``): their width says how much of a head is
     rotated, ``pairing`` which elements go together.  ``value_dim``: the value heads' own size (then a row may
-    also hold further columns behind the heads, which are left alone)."""
+    also hold further columns behind the heads, which are left alone).  ``queries_only``: the rows hold the query
+    heads (and perhaps further columns) but no key and value heads: a layer that reads another layer's cache."""
     planes = qkv.shape[0] if qkv.dim() == 3 else 1
     rows, width = qkv.shape[-2:]
     kind = out_dtype or qkv.dtype
@@ -225,7 +250,10 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim:
     general = value_dim is not None
     value_dim = head_dim if value_dim is None else int(value_dim)
     heads_width = (q_heads + kv_heads) * head_dim + kv_heads * value_dim
-    if width != heads_width and not (general and width > heads_width and planes == 1):
+    if queries_only:
+        if write_cache or planes != 1 or width < q_heads * head_dim:
+            raise KernelError(f"qk_norm_rope_write: rows of {width} with query heads only ({q_heads}*{head_dim}) write no cache")
+    elif width != heads_width and not (general and width > heads_width and planes == 1):
         raise KernelError(f"qk_norm_rope_write: width {width} is not ({q_heads}+{kv_heads})*{head_dim}+{kv_heads}*{value_dim}")
     if out is None:
         out = torch.empty((rows, q_heads * head_dim), dtype=kind, device=qkv.device)
@@ -268,22 +296,26 @@ def _strided_rows(t: Optional[torch.Tensor], what: str, rows: int, columns: int,
 
 def attention_rows(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
                    row_entry: torch.Tensor, block_table: torch.Tensor, q_heads: int, scale: float,
-                   window: int = 0, out: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Each query row attends its request's cached keys up to its own position.  The result has the values'
+                   window: int = 0, out: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                   keep_first: int = 0, gate_each: bool = False) -> torch.Tensor:
+    """Each query row attends its request's cached keys up to its own position (the last ``window`` of them,
+    and, whatever the window, those at positions below ``keep_first``).  The result has the values'
     size a head.  ``gate``: float32 ``[rows, >= q_heads]`` (a view into a wider row is fine, unit stride along the
-    heads): head h of row r is multiplied by sigmoid(gate[r, h])."""
+    heads): head h of row r is multiplied by sigmoid(gate[r, h]); with ``gate_each`` the gate holds a value for
+    every element of the result, ``[rows, >= q_heads * value_dim]``."""
     rows = q.shape[0]
     pages, kv_heads, page_tokens, head_dim, value_dim = cache_dims_kv(k_pool, v_pool)
     if q.shape[1] != q_heads * head_dim:
         raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
     if out is None:
         out = torch.empty((rows, q_heads * value_dim), dtype=q.dtype, device=q.device)
-    gate_at, gate_stride = _strided_rows(gate, "attention gate", rows, q_heads)
-    call("leone_attention_rows", _dev(q, "attention q"), _dev(out, "attention out", q.dtype, (rows, q_heads * value_dim)),
+    gate_at, gate_stride = _strided_rows(gate, "attention gate", rows, q_heads * value_dim if gate_each else q_heads)
+    call("leone_attention_rows_kept", _dev(q, "attention q"), _dev(out, "attention out", q.dtype, (rows, q_heads * value_dim)),
          _dev(k_pool, "k pool", q.dtype), _dev(v_pool, "v pool", q.dtype), _code(q, "attention q"),
          _dev(positions, "positions", torch.int32, (rows,)), _dev(row_entry, "row map", torch.int32, (rows,)),
          _dev(block_table, "block table", torch.int32), block_table.shape[1], rows, q_heads, kv_heads, head_dim,
-         value_dim, page_tokens, float(scale), int(window), gate_at, gate_stride, _stream())
+         value_dim, page_tokens, float(scale), int(window), gate_at, gate_stride, int(keep_first),
+         1 if (gate_each and gate is not None) else 0, _stream())
     return out
 
 
@@ -589,7 +621,7 @@ def drop_streamed_copies() -> None:
 
 
 def gemm_fused(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-               residual: Optional[torch.Tensor] = None, gated: bool = False, next_norm=None):
+               residual: Optional[torch.Tensor] = None, gated: bool = False, next_norm=None, activation: str = "silu"):
     """The product for at most 16 rows with its neighbours folded in: ``x`` may be ``NormedRows`` or
     ``PreparedRows``; with ``residual`` the product is added into that float32 tensor and None is returned;
     with ``gated`` the weight is an interleaved gate/up weight and silu(gate) * up comes out.  With
@@ -613,7 +645,9 @@ def gemm_fused(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
             operand = torch.empty((m, n), dtype=torch.bfloat16, device=weight.device)
             squares = torch.empty((m, -(-n // 16)), dtype=torch.float32, device=weight.device)
     elif gated:
-        out, mode, out_dtype = torch.empty((m, n // 2), dtype=torch.bfloat16, device=weight.device), 2, torch.bfloat16
+        # mode 4: the gated output with the tanh form of gelu on the gate
+        out, mode, out_dtype = (torch.empty((m, n // 2), dtype=torch.bfloat16, device=weight.device),
+                                4 if _gate_code(activation) == 1 else 2, torch.bfloat16)
     else:
         out, mode = torch.empty((m, n), dtype=out_dtype, device=weight.device), 0
     if prepared:
@@ -699,7 +733,8 @@ def rows_ways(m: int, waves: int) -> int:
 
 def gemm_rows(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
               residual: Optional[torch.Tensor] = None, gated: bool = False, splits: Optional[int] = None,
-              waves: Optional[int] = None, may_split: bool = True, ways: Optional[int] = None) -> Optional[torch.Tensor]:
+              waves: Optional[int] = None, may_split: bool = True, ways: Optional[int] = None,
+              activation: str = "silu") -> Optional[torch.Tensor]:
     """The weight-streaming product for up to ROWS_MAX rows of bfloat16 ``x``.  With ``residual`` and one
     range of K the product is added into that float32 tensor (None returned); with ``gated`` the weight is
     an interleaved gate/up weight and silu(gate) * up comes out.  With more than one range of K (``splits``;
@@ -735,7 +770,8 @@ def gemm_rows(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = to
         out, mode, kind = residual, 1, torch.float32
         _dev(out, "gemm_rows stream", torch.float32, (m, n))
     elif gated:
-        out, mode, kind = torch.empty((m, n // 2), dtype=torch.bfloat16, device=weight.device), 2, torch.bfloat16
+        out, mode, kind = (torch.empty((m, n // 2), dtype=torch.bfloat16, device=weight.device),
+                           4 if _gate_code(activation) == 1 else 2, torch.bfloat16)
     else:
         out, mode, kind = torch.empty((m, n), dtype=out_dtype, device=weight.device), 0, out_dtype
     tiles = streamed_copy(weight) if _streamed else None
@@ -887,11 +923,12 @@ def _library_product(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dty
 
 def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
            residual: Optional[torch.Tensor] = None, gated: bool = False,
-           planes_ok: bool = False, next_norm=None):
+           planes_ok: bool = False, next_norm=None, activation: str = "silu"):
     """x[R,K] . weight[N,K]^T, with optional neighbours.
 
     ``x`` is a tensor or ``NormedRows`` (a norm still to be done).  ``gated``: the weight is an
-    interleaved gate/up weight and the result is silu(gate) * up, ``[R, N/2]``.  ``residual``: the caller
+    interleaved gate/up weight and the result is act(gate) * up, ``[R, N/2]``, act being silu or what
+    ``activation`` names (``GATE_ACTIVATIONS``).  ``residual``: the caller
     wants the product added into this float32 tensor; if the kernel in use can do that, it does and None
     is returned, otherwise the product is returned for the caller to add later, as float32 ``[R, N]`` or
     as a stack of planes ``[p, R, N]`` whose sum is meant (``add_rmsnorm`` takes either).
@@ -921,11 +958,12 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         if next_norm is not None and (residual is None or not prepared_fits(rows, weight.shape[0])
                                       or next_norm[2] != torch.bfloat16):
             next_norm = None
-        return gemm_fused(x, weight, out_dtype, residual, gated, next_norm)
+        return gemm_fused(x, weight, out_dtype, residual, gated, next_norm, activation=activation)
     x = materialize(x)
     if dtype == torch.bfloat16 and weight.is_cuda and k % 8 == 0 and rows <= ROWS_MAX \
             and (not gated or weight.shape[0] % 16 == 0):
-        return gemm_rows(x, weight, out_dtype, residual, gated, may_split=planes_ok or residual is not None)
+        return gemm_rows(x, weight, out_dtype, residual, gated, may_split=planes_ok or residual is not None,
+                         activation=activation)
     if dtype == torch.float32:
         if out_dtype != torch.float32:
             raise KernelError("linear: the float32 path produces float32")
@@ -950,7 +988,7 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
             y = _library_product(x, weight, torch.bfloat16, None)
         if out_dtype != y.dtype:
             y = y.to(out_dtype)
-    return swiglu(y) if gated else y
+    return swiglu(y, activation=activation) if gated else y
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:
@@ -1380,4 +1418,92 @@ def delta_scan(qkv: torch.Tensor, columns: dict, beta: torch.Tensor, step_size: 
         walk(plan["again"], work, None, no_input=True, accumulate=True)
         if plan["short"].shape[0]:
             walk(plan["short"], state, state if write_state else None)
+    return out
+
+
+# ---- a norm behind the sublayer, routed experts ----------------------------------------------------------------
+def add_normed(x: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional[torch.Tensor], eps: float,
+               out_dtype: Optional[torch.dtype] = None, then: Optional[tuple] = None,
+               rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x += rmsnorm(delta) * gain in the float32 stream (``delta`` float32 ``[n, hidden]`` or planes ``[p, n, hidden]``
+    whose sum, in order, is meant; None: nothing is added).  What comes back: with ``out_dtype`` the new rows of
+    the stream in that type (what the next sublayer's products read); with ``then = (gain2, eps2, dtype)`` instead
+    rmsnorm(x) * gain2 of the new rows, of the rows ``rows`` (int32 indices) only if given, and then the stream
+    itself is left as it was."""
+    n, hidden = x.shape
+    if delta is not None and delta.dtype != torch.float32:
+        delta = delta.float()
+    stacked = delta is not None and delta.dim() == 3
+    planes = delta.shape[0] if stacked else 1
+    if rows is not None and then is None:
+        raise KernelError("add_normed: picked rows come with a second norm")
+    n_out = n if rows is None else rows.numel()
+    kind = then[2] if then is not None else out_dtype
+    if delta is None and kind is None:
+        return None
+    if delta is None and then is None and kind == torch.float32:
+        return x                                   # nothing to add, nothing to convert
+    same = then is None and kind == torch.float32          # the stream itself is what the next products read
+    y = torch.empty((n_out, hidden), dtype=kind, device=x.device) if (kind is not None and not same) else None
+    call("leone_add_normed", _dev(x, "stream", torch.float32),
+         _dev(delta, "delta", torch.float32, (planes, n, hidden) if stacked else (n, hidden)), planes, n * hidden,
+         _dev(gain, "gain", None, (hidden,)) if delta is not None else 0,
+         _code(gain, "gain") if delta is not None else F32, float(eps),
+         _dev(y, "rows out"), _CODES[kind] if kind is not None else F32,
+         _dev(then[0], "second gain", None, (hidden,)) if then is not None else 0,
+         _code(then[0], "second gain") if then is not None else F32, float(then[1]) if then is not None else 0.0,
+         _dev(rows, "rows", torch.int32) if rows is not None else 0, n_out, hidden, _stream())
+    return x if same else y
+
+
+def route_topk(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, group_count: int = 1,
+               group_keep: int = 1) -> tuple:
+    """The router's choice for every row of float32 ``logits [rows, outputs]``: scores softmax(logits); choice scores
+    with ``correction`` added; the outputs form ``group_count`` equal groups of neighbours of which the
+    ``group_keep`` with the best choice score stay open; the ``top`` best open outputs win.  Returns their
+    indices (int32 ``[rows, top]``, best first) and their scores over the winners' sum (float32)."""
+    rows, total = logits.shape
+    if total > library().leone_route_max_outputs():
+        raise KernelError(f"route_topk: {total} router outputs, the kernel takes {library().leone_route_max_outputs()}")
+    chosen = torch.empty((rows, top), dtype=torch.int32, device=logits.device)
+    weight = torch.empty((rows, top), dtype=torch.float32, device=logits.device)
+    call("leone_route_topk", _dev(logits, "router logits", torch.float32),
+         _dev(correction, "router correction", None, (total,)), _code(correction, "router correction") if correction is not None else F32,
+         _dev(chosen, "chosen"), _dev(weight, "weights"), rows, total, int(top), int(group_count), int(group_keep), _stream())
+    return chosen, weight
+
+
+def routed_experts(x: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, w_gate_up: torch.Tensor,
+                   w_down: torch.Tensor, activation: str = "silu", extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Every row through the experts chosen for it: float32 ``[rows, hidden]`` = sum over a row's places of
+    weight * W_down[e] (act(W_gate[e] x) * (W_up[e] x)), in the places' order; a chosen index from the number of
+    experts on stands for an expert that hands the row on as it is; ``extra`` (float32 ``[rows, hidden]``) is added.
+    ``w_gate_up`` is ``[experts, 2, ff, hidden]`` (gate rows, then up rows), ``w_down`` ``[experts, hidden, ff]``, both
+    of ``x``'s type.  Nothing here depends on the choice except through device arrays."""
+    rows, hidden = x.shape
+    top = chosen.shape[1]
+    experts, two, ff, k = w_gate_up.shape
+    if two != 2 or k != hidden or tuple(w_down.shape) != (experts, hidden, ff) or w_gate_up.dtype != x.dtype or w_down.dtype != x.dtype:
+        raise KernelError(f"routed_experts: matrices {tuple(w_gate_up.shape)} and {tuple(w_down.shape)} of {w_gate_up.dtype} "
+                          f"do not fit rows {tuple(x.shape)} of {x.dtype}")
+    pairs = rows * top
+    tile = library().leone_moe_tile_pairs()
+    max_tiles = min(pairs, pairs // tile + experts)
+    device = x.device
+    tile_expert = torch.empty((max_tiles,), dtype=torch.int32, device=device)
+    tile_pairs = torch.empty((max_tiles, tile), dtype=torch.int32, device=device)
+    call("leone_moe_plan", _dev(chosen, "chosen", torch.int32, (rows, top)), pairs, experts, _dev(tile_expert, "tiles"),
+         _dev(tile_pairs, "tile pairs"), max_tiles, _stream())
+    hidden_act = torch.empty((pairs, ff), dtype=x.dtype, device=device)
+    call("leone_moe_product", _dev(x, "routed rows"), _dev(w_gate_up, "expert gate/up"), _dev(hidden_act, "expert hidden"), 0,
+         _code(x, "routed rows"), 1, _dev(tile_expert, "tiles"), _dev(tile_pairs, "tile pairs"), max_tiles, top, ff, hidden,
+         _gate_code(activation), _stream())
+    pair_out = torch.empty((pairs, hidden), dtype=torch.float32, device=device)
+    call("leone_moe_product", _dev(hidden_act, "expert hidden"), _dev(w_down, "expert down"), _dev(pair_out, "pair results"),
+         _dev(weight, "weights", torch.float32, (rows, top)), _code(x, "routed rows"), 0, _dev(tile_expert, "tiles"),
+         _dev(tile_pairs, "tile pairs"), max_tiles, top, hidden, ff, 0, _stream())
+    out = torch.empty((rows, hidden), dtype=torch.float32, device=device)
+    call("leone_moe_combine", _dev(pair_out, "pair results"), _dev(chosen, "chosen"), _dev(weight, "weights"),
+         _dev(x, "routed rows"), _code(x, "routed rows"), _dev(extra, "extra", torch.float32, (rows, hidden)),
+         _dev(out, "routed out"), rows, top, experts, hidden, _stream())
     return out

@@ -68,6 +68,15 @@ _PROTOTYPES = {
     "leone_outer_chain": [P, c_int, P, ctypes.c_long, P, P, ctypes.c_long, ctypes.c_long, c_int, c_int, c_int, P],
     "leone_delta_scan": [P, ctypes.c_long, c_int, c_int, c_int, P, ctypes.c_long, P, ctypes.c_long, P, P, c_int, c_float,
                          c_float, c_int, c_int, P, c_int, P, ctypes.c_long, P, ctypes.c_long, P, P, c_int, c_int, c_int, c_int, P],
+    "leone_embed_placed": [P, c_int, P, P, c_int, c_int, c_int, c_float, P, P, c_int, P],
+    "leone_glu": [P, P, c_int, c_int, c_int, c_int, P],
+    "leone_add_normed": [P, P, c_int, ctypes.c_long, P, c_int, c_float, P, c_int, P, c_int, c_float, P, c_int, c_int, P],
+    "leone_attention_rows_kept": [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                                  c_int, P, ctypes.c_long, c_int, c_int, P],
+    "leone_route_topk": [P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "leone_moe_plan": [P, c_int, c_int, P, P, c_int, P],
+    "leone_moe_product": [P, P, P, P, c_int, c_int, P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "leone_moe_combine": [P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, P],
     "leone_delta_chain": [P, c_int, P, ctypes.c_long, P, P, ctypes.c_long, c_int, c_int, c_int, c_int, P],
 }
 
@@ -106,6 +115,10 @@ def library() -> ctypes.CDLL:
             lib.leone_gemm_rows_max_rows.argtypes = []
             lib.leone_gemm_rows_chunk.restype = c_int
             lib.leone_gemm_rows_chunk.argtypes = [c_int]
+            lib.leone_moe_tile_pairs.restype = c_int
+            lib.leone_moe_tile_pairs.argtypes = []
+            lib.leone_route_max_outputs.restype = c_int
+            lib.leone_route_max_outputs.argtypes = []
             lib.leone_library_product_available.restype = c_int
             lib.leone_library_product_available.argtypes = []
             lib.leone_library_product_tuned.restype = c_int

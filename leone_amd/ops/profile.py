@@ -47,6 +47,14 @@ OPERATIONS = {
     "leone_exp_gates": "exp gates",
     "leone_delta_scan": "delta scan",
     "leone_delta_chain": "delta scan",
+    "leone_embed_placed": "embed",
+    "leone_glu": "swiglu",
+    "leone_add_normed": "norm",
+    "leone_attention_rows_kept": "attention",
+    "leone_route_topk": "router",
+    "leone_moe_plan": "router",
+    "leone_moe_product": "experts",
+    "leone_moe_combine": "experts",
 }
 LIBRARY_PRODUCT = "gemm library"
 ORDER = ["embed", "norm", "gemv fused", "gemm rows", LIBRARY_PRODUCT, "gemm f32", "qknorm rope kv", "attention", "swiglu",

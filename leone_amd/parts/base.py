@@ -79,6 +79,7 @@ class KvNeed:
     window: Optional[int] = None   # only the last `window` positions are ever read
     page_tokens: Optional[int] = None   # tokens a page of this group holds; None: the engine's choice
     value_dim: Optional[int] = None     # size of a value vector; None: the keys' size
+    keep_first: int = 0                 # with a window: the first positions stay readable too (their pages are kept)
 
     paged = True
 

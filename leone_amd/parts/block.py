@@ -172,3 +172,71 @@ class SandwichBlock(Part):
             return pending
         h = self._read(self.norm2, self.conv2, x, pending, step, cache.get("conv2"))
         return ops.NormedDelta(self.feed_forward.forward(h, step), self.norm2b)
+
+
+@BLOCKS.register("postnorm")
+class PostNormBlock(Part):
+    """The norms stand behind the sublayers, which read the stream itself:
+
+        x <- x + norm1(mixer(x));   x <- x + norm2(feed_forward(x))
+
+    The second sublayer is there only if ``feed_forward`` is given.  Parameters: ``mixer``, ``norm1`` and optionally
+    ``feed_forward``, ``norm2`` (part specs); the norms are RMS norms.  The sublayers hand back float32.  A norm
+    behind a sublayer, the residual sum and the rows of the stream in the type the next sublayer's products read
+    are one kernel (``ops.add_normed``); the block's last norm is left to whoever runs next (``ops.NormedDelta``):
+    the next block of this kind, or the model's final norm, which does both norms and the sum in one kernel.
+    """
+
+    def __init__(self, spec: PartSpec, **context):
+        self.mixer = MIXERS.build(spec["mixer"], **context)
+        self.norm1 = NORMS.build(spec["norm1"], **context)
+        self.feed_forward = FEED_FORWARDS.build(spec["feed_forward"], **context) if spec.get("feed_forward") is not None else None
+        self.norm2 = NORMS.build(spec["norm2"], **context) if spec.get("norm2") is not None else None
+        if self.feed_forward is not None and self.norm2 is None:
+            raise ValueError("a postnorm block with a feed-forward needs norm2")
+        for norm in (self.norm1, self.norm2):
+            if norm is not None and not hasattr(norm, "add_behind"):
+                raise ValueError("the norms of a postnorm block must be able to stand behind a sublayer (add_behind)")
+
+    def parts(self):
+        return tuple(part for part in (self.mixer, self.norm1, self.feed_forward, self.norm2) if part is not None)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", False) for part in self.parts())
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for part in self.parts() for s in part.tensor_specs()]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for part in self.parts():
+            part.bind(tensors)
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [w for part in self.parts() if hasattr(part, "streamed_weights") for w in part.streamed_weights()]
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def row_tilings(self):
+        return [part.row_tiling() for part in self.parts() if hasattr(part, "row_tiling")]
+
+    @staticmethod
+    def _take_in(x: torch.Tensor, pending, step: StepContext) -> torch.Tensor:
+        """Adds what the block before left to be added and returns the stream's rows as the products read them."""
+        if isinstance(pending, ops.PreparedRows):
+            pending = None                        # its product has added into the stream already
+        if isinstance(pending, ops.NormedDelta) and hasattr(pending.norm, "add_behind"):
+            return pending.norm.add_behind(x, pending.rows, step.dtype)
+        if pending is not None:
+            delta = pending.materialize() if isinstance(pending, ops.NormedDelta) else pending
+            x.add_(delta.sum(dim=0) if delta.dim() == 3 else delta)
+        return ops.add_normed(x, None, None, 0.0, out_dtype=step.dtype)
+
+    def forward(self, x: torch.Tensor, pending, step: StepContext, cache: Optional[CacheView]):
+        h = self._take_in(x, pending, step)
+        mixed = self.mixer.forward(h, step, cache)
+        if self.feed_forward is None:
+            return ops.NormedDelta(mixed, self.norm1)
+        h = self.norm1.add_behind(x, mixed, step.dtype)
+        return ops.NormedDelta(self.feed_forward.forward(h, step), self.norm2)

@@ -6,7 +6,7 @@ from typing import Dict, List, Optional
 import torch
 
 from .. import ops
-from ..weights.loader import MATRIX, TensorSpec
+from ..weights.loader import MATRIX, VECTOR, TensorSpec
 from .base import FEED_FORWARDS, Part, PartSpec
 from .context import StepContext
 
@@ -17,6 +17,8 @@ class SwiGluMlp(Part):
 
     Reference: crates/leone/src/runtime.rs:9283-9319, crates/leone/src/cpu.rs:892-907.
     Parameters: ``hidden``, ``intermediate`` and tensor names ``gate``, ``up``, ``down``.
+    Optional: ``activation`` (what stands on the gate instead of silu, a key of ``ops.GATE_ACTIVATIONS``),
+    ``float_output`` (what is handed back comes in float32 whatever the engine's type).
     """
 
     graph_safe = True
@@ -26,6 +28,10 @@ class SwiGluMlp(Part):
         self.hidden = int(p["hidden"])
         self.intermediate = int(p["intermediate"])
         self.names = {k: p[k] for k in ("gate", "up", "down")}
+        self.activation = str(p.get("activation") or "silu")
+        if self.activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"unknown gate activation {self.activation!r}; known: {', '.join(ops.GATE_ACTIVATIONS)}")
+        self.float_output = bool(p.get("float_output", False))
         self.w_gate_up = self.w_down = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -56,8 +62,9 @@ class SwiGluMlp(Part):
     def forward(self, y, step: StepContext, residual: Optional[torch.Tensor] = None, next_norm=None):
         """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned),
         and with ``next_norm`` the norm that follows may come back prepared (see ``ops.linear``)."""
-        activated = ops.linear(y, self.w_gate_up, gated=True)
-        return ops.linear(activated, self.w_down, residual=residual, next_norm=next_norm)
+        activated = ops.linear(y, self.w_gate_up, gated=True, activation=self.activation)
+        return ops.linear(activated, self.w_down, residual=residual, next_norm=next_norm,
+                          out_dtype=torch.float32 if self.float_output else None)
 
 
 @FEED_FORWARDS.register("relu2")
@@ -85,3 +92,79 @@ class ReluSquaredMlp(Part):
 
     def forward(self, y: torch.Tensor, step: StepContext) -> torch.Tensor:
         return ops.linear(ops.relu_squared(ops.linear(y, self.w_up)), self.w_down, out_dtype=torch.float32)
+
+
+@FEED_FORWARDS.register("routed_glu")
+class RoutedGluMlp(Part):
+    """A mixture of small gated feed-forwards of which a router picks ``top`` for every row.
+
+    Router logits z = W_router y in float; scores s = softmax(z) over all router outputs; a row's choice scores are
+    s + ``correction``; the outputs form ``group_count`` equal groups of neighbours, a group's score is its best
+    choice score, and only outputs of the ``group_keep`` best groups can be chosen; the ``top`` best choice scores
+    win and weigh in with s over the winners' sum.  The first ``experts`` outputs are experts
+    down_e(act(gate_e y) * (up_e y)); the ``identity`` outputs behind them hand y itself on.  A ``shared`` feed-forward
+    (a part spec, optional) runs for every row and is added.  The result is float32.
+
+    Parameters: ``hidden``, ``experts``, ``identity``, ``top``, ``group_count``, ``group_keep``, ``intermediate``,
+    ``activation`` (a key of ``ops.GATE_ACTIVATIONS``), tensor names ``router`` ``[experts + identity, hidden]``,
+    ``correction`` ``[experts + identity]`` (None: no correction) and ``expert`` (a pattern with ``{e}``:
+    ``expert.format(e=3) + ".gate"`` and so on), ``shared``.
+
+    The choice lives on the device only: which rows go to which expert is worked out there, and the grids do not
+    depend on it, so a recorded step replays with other choices.
+    """
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, **context):
+        p = spec.params
+        self.hidden, self.intermediate = int(p["hidden"]), int(p["intermediate"])
+        self.experts, self.identity, self.top = int(p["experts"]), int(p.get("identity") or 0), int(p["top"])
+        self.group_count, self.group_keep = int(p.get("group_count") or 1), int(p.get("group_keep") or 1)
+        self.activation = str(p.get("activation") or "silu")
+        self.total = self.experts + self.identity
+        if self.top > self.total or self.total % self.group_count or not 1 <= self.group_keep <= self.group_count:
+            raise ValueError(f"a router of {self.total} outputs cannot choose {self.top} from {self.group_keep} of "
+                             f"{self.group_count} equal groups")
+        if self.activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"unknown gate activation {self.activation!r}; known: {', '.join(ops.GATE_ACTIVATIONS)}")
+        self.router_name, self.correction_name, self.expert_name = p["router"], p.get("correction"), p["expert"]
+        self.shared = FEED_FORWARDS.build(p["shared"], **context) if p.get("shared") is not None else None
+        self.w_router = self.correction = self.w_gate_up = self.w_down = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = [TensorSpec(self.router_name, (self.total, self.hidden), MATRIX)]
+        if self.correction_name:
+            specs.append(TensorSpec(self.correction_name, (self.total,), VECTOR))
+        for e in range(self.experts):
+            name = self.expert_name.format(e=e)
+            specs += [TensorSpec(name + ".gate", (self.intermediate, self.hidden), MATRIX),
+                      TensorSpec(name + ".up", (self.intermediate, self.hidden), MATRIX),
+                      TensorSpec(name + ".down", (self.hidden, self.intermediate), MATRIX)]
+        return specs + (self.shared.tensor_specs() if self.shared is not None else [])
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.w_router = tensors.pop(self.router_name).contiguous()
+        self.correction = tensors.pop(self.correction_name).contiguous() if self.correction_name else None
+        names = [self.expert_name.format(e=e) for e in range(self.experts)]
+        # all experts side by side: [experts, 2, ff, hidden] (gate rows, then up rows) and [experts, hidden, ff]
+        self.w_gate_up = torch.stack([torch.stack([tensors.pop(n + ".gate"), tensors.pop(n + ".up")]) for n in names]).contiguous()
+        self.w_down = torch.stack([tensors.pop(n + ".down") for n in names]).contiguous()
+        if self.shared is not None:
+            self.shared.bind(tensors)
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return self.shared.streamed_weights() if self.shared is not None else []
+
+    def forward(self, y: torch.Tensor, step: StepContext) -> torch.Tensor:
+        y = ops.materialize(y)
+        logits = ops.linear(y, self.w_router, out_dtype=torch.float32)
+        chosen, weight = ops.route_topk(logits, self.correction, self.top, self.group_count, self.group_keep)
+        extra = None
+        if self.shared is not None:
+            extra = self.shared.forward(y, step)
+            if extra.dim() == 3:
+                extra = extra.sum(dim=0)
+            if extra.dtype != torch.float32:
+                extra = extra.float()
+        return ops.routed_experts(y, chosen, weight, self.w_gate_up, self.w_down, self.activation, extra=extra)

@@ -32,6 +32,12 @@ class GqaAttention(Part):
     of a head have this size instead of ``head_dim``), ``gate`` (tensor name ``[q_heads, hidden]``: head h's
     result is multiplied by sigmoid(gate y)_h before the output projection), ``float_output`` (the output
     projection's result comes in float32 whatever the engine's type).
+    ``gate_each`` (with ``gate``): the gate is ``[q_heads * value_dim, hidden]``, one value for every element of
+    the heads' results.  ``keep_first`` (with ``window``): keys at positions below it stay in sight whatever the
+    window, at their own positions.  ``shared_kv``: the layer has no key and value projections (and no key norm)
+    and reads the cache another layer writes (its run names that layer's cache slot and does not write).
+    ``retain_window`` / ``retain_first``: what the cache must keep if other layers with wider masks read it too
+    (by default this layer's own ``window`` and ``keep_first``; ``retain_window`` 0: everything).
     """
 
     graph_safe = True
@@ -47,23 +53,31 @@ class GqaAttention(Part):
         self.qk_norm_eps = p.get("qk_norm_eps")
         self.window = p.get("window")
         self.scale = float(p.get("scale", 1.0 / math.sqrt(self.head_dim)))
-        self.names = {k: p[k] for k in ("q", "k", "v", "o")}
+        self.shared_kv = bool(p.get("shared_kv", False))
+        self.names = {k: p[k] for k in (("q", "o") if self.shared_kv else ("q", "k", "v", "o"))}
+        self.keep_first = int(p.get("keep_first") or 0) if self.window else 0
+        self.gate_each = bool(p.get("gate_each", False))
+        self.retain_window = self.window if "retain_window" not in p else (p["retain_window"] or None)
+        self.retain_first = int(p.get("retain_first", self.keep_first) or 0)
         self.value_dim = int(p.get("value_dim") or self.head_dim)
         self.float_output = bool(p.get("float_output", False))
         if p.get("gate"):
             self.names["gate"] = p["gate"]
         # a value size of its own or a gate: the projection carries more than q, k and v of one size
-        self.general = self.value_dim != self.head_dim or "gate" in self.names
+        self.general = self.value_dim != self.head_dim or "gate" in self.names or self.shared_kv
         if self.qk_norm_eps is not None:
-            self.names.update(q_norm=p["q_norm"], k_norm=p["k_norm"])
+            self.names.update(q_norm=p["q_norm"])
+            if not self.shared_kv:
+                self.names.update(k_norm=p["k_norm"])
         self.position = (positions or {}).get(p.get("position")) if p.get("position") else None
         if p.get("position") and self.position is None:
             raise ValueError(f"attention names position part {p.get('position')!r}, which the model does not define")
         self.w_qkv = self.w_o = self.q_gain = self.k_gain = None
 
     def cache_need(self) -> KvNeed:
-        return KvNeed(self.kv_heads, self.head_dim, self.window,
-                      value_dim=self.value_dim if self.value_dim != self.head_dim else None)
+        return KvNeed(self.kv_heads, self.head_dim, self.retain_window,
+                      value_dim=self.value_dim if self.value_dim != self.head_dim else None,
+                      keep_first=self.retain_first if self.retain_window else 0)
 
     def row_tiling(self) -> RowTiling:
         """The tiles of the prompt-attention kernel."""
@@ -71,27 +85,33 @@ class GqaAttention(Part):
 
     def tensor_specs(self) -> List[TensorSpec]:
         qw, kvw = self.q_heads * self.head_dim, self.kv_heads * self.head_dim
-        specs = [TensorSpec(self.names["q"], (qw, self.hidden), MATRIX),
-                 TensorSpec(self.names["k"], (kvw, self.hidden), MATRIX),
-                 TensorSpec(self.names["v"], (self.kv_heads * self.value_dim, self.hidden), MATRIX),
-                 TensorSpec(self.names["o"], (self.hidden, self.q_heads * self.value_dim), MATRIX)]
+        specs = [TensorSpec(self.names["q"], (qw, self.hidden), MATRIX)]
+        if not self.shared_kv:
+            specs += [TensorSpec(self.names["k"], (kvw, self.hidden), MATRIX),
+                      TensorSpec(self.names["v"], (self.kv_heads * self.value_dim, self.hidden), MATRIX)]
+        specs.append(TensorSpec(self.names["o"], (self.hidden, self.q_heads * self.value_dim), MATRIX))
         if "gate" in self.names:
-            specs.append(TensorSpec(self.names["gate"], (self.q_heads, self.hidden), MATRIX))
+            gates = self.q_heads * self.value_dim if self.gate_each else self.q_heads
+            specs.append(TensorSpec(self.names["gate"], (gates, self.hidden), MATRIX))
         if self.qk_norm_eps is not None:
-            specs += [TensorSpec(self.names["q_norm"], (self.head_dim,), VECTOR),
-                      TensorSpec(self.names["k_norm"], (self.head_dim,), VECTOR)]
+            specs.append(TensorSpec(self.names["q_norm"], (self.head_dim,), VECTOR))
+            if not self.shared_kv:
+                specs.append(TensorSpec(self.names["k_norm"], (self.head_dim,), VECTOR))
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         # One product for q, k and v: a pure re-layout of the three matrices.
-        fused = [tensors.pop(self.names["q"]), tensors.pop(self.names["k"]), tensors.pop(self.names["v"])]
+        fused = [tensors.pop(self.names["q"])]
+        if not self.shared_kv:
+            fused += [tensors.pop(self.names["k"]), tensors.pop(self.names["v"])]
         if "gate" in self.names:
             fused.append(tensors.pop(self.names["gate"]))      # the heads' gates ride along as further columns
         self.w_qkv = torch.cat(fused, dim=0).contiguous()
         self.w_o = tensors.pop(self.names["o"]).contiguous()
         if self.qk_norm_eps is not None:
             self.q_gain = tensors.pop(self.names["q_norm"]).contiguous()
-            self.k_gain = tensors.pop(self.names["k_norm"]).contiguous()
+            # a layer without keys of its own never normalises one; the kernels want the two gains together
+            self.k_gain = self.q_gain if self.shared_kv else tensors.pop(self.names["k_norm"]).contiguous()
             if self.q_gain.dtype != self.k_gain.dtype:
                 self.q_gain, self.k_gain = self.q_gain.float(), self.k_gain.float()
 
@@ -114,11 +134,12 @@ class GqaAttention(Part):
             q = ops.qk_norm_rope_write(proj, self.q_heads, self.kv_heads, self.head_dim, self.q_gain, self.k_gain,
                                        self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, rotation.cos, rotation.sin,
                                        step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
-                                       write_cache=cache.writes, out_dtype=step.dtype, pairing=rotation.pairing,
-                                       value_dim=self.value_dim)
+                                       write_cache=cache.writes and not self.shared_kv, out_dtype=step.dtype,
+                                       pairing=rotation.pairing, value_dim=self.value_dim, queries_only=self.shared_kv)
             gate = None
             if "gate" in self.names:
-                gate = proj[:, (self.q_heads + self.kv_heads) * self.head_dim + self.kv_heads * self.value_dim:]
+                gate = proj[:, self.q_heads * self.head_dim:] if self.shared_kv else \
+                    proj[:, (self.q_heads + self.kv_heads) * self.head_dim + self.kv_heads * self.value_dim:]
             attended = self._attend(q, step, cache, gate)
             return ops.linear(attended, self.w_o, out_dtype=out_dtype, residual=residual, next_norm=next_norm)
         qkv = ops.linear(y, self.w_qkv, planes_ok=True)
@@ -150,12 +171,17 @@ class GqaAttention(Part):
         ``prompt`` (portions of at least ``ops.PREFILL_MIN_ROWS`` rows): "flash" (the matrix-core prompt
         kernel), else what single tokens get."""
         group = self.q_heads // self.kv_heads
-        if self.value_dim != self.head_dim or not ops.decode_attention_supported(dtype, self.head_dim, page_tokens, group, max_blocks):
+        if self._rows_only() or not ops.decode_attention_supported(dtype, self.head_dim, page_tokens, group, max_blocks):
             return {"decode": "rows", "prompt": "rows"}
         rotation = rotation_of(self.position)
         projected = not self.general and ops.decode_projected_supported(self.head_dim, rotation.rotary_dim, rotation.pairing)
         return {"decode": "projected" if projected else "split_kv",
                 "prompt": "flash" if ops.prefill_attention_supported(dtype, self.head_dim, page_tokens, max_blocks) else "split_kv"}
+
+    def _rows_only(self) -> bool:
+        """What the matrix-core kernels are not built for: values of another size than the keys, kept first keys
+        beside a window, a gate for every element."""
+        return self.value_dim != self.head_dim or bool(self.window and self.keep_first) or self.gate_each
 
     def _attend(self, q: torch.Tensor, step: StepContext, cache: KvCacheView, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Long prompt portions through the prompt kernel, the other rows through the split-KV kernel; the
@@ -164,10 +190,11 @@ class GqaAttention(Part):
         window = int(self.window or 0)
         group = self.q_heads // self.kv_heads
         max_blocks = cache.block_table.shape[1]
-        if self.value_dim != self.head_dim or \
+        if self._rows_only() or \
                 not ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens, group, max_blocks):
             return ops.attention_rows(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
-                                      cache.block_table, self.q_heads, self.scale, window, gate=gate)
+                                      cache.block_table, self.q_heads, self.scale, window, gate=gate,
+                                      keep_first=self.keep_first, gate_each=self.gate_each)
         first = 0
         out = torch.empty_like(q)
         tiled = step.tiled.get(self.row_tiling())

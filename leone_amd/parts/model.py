@@ -40,6 +40,7 @@ class ModelSpec:
     ignore_tensors: Sequence[str] = ()              # names a file may hold that the model does not use
     embedding_scale: Optional[float] = None         # the stream starts as table row * scale
     logit_cap: Optional[float] = None               # logits = cap * tanh(logits / cap)
+    position_table: Optional[str] = None            # tensor name [max_positions, hidden]: a learned vector a position, added to the token's
 
 
 def default_schedule(n_layers: int) -> List[LayerRun]:
@@ -63,6 +64,7 @@ class DecoderModel:
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"schedule names layer {run.layer}, the model has {len(self.layers)}")
         self.embedding: Optional[torch.Tensor] = None
+        self.position_table: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
         self.streamed_copy_bytes: Optional[int] = None    # None: not decided yet (``keep_streamed_copies``)
 
@@ -75,6 +77,8 @@ class DecoderModel:
     # ---- weights -------------------------------------------------------------
     def tensor_specs(self) -> List[TensorSpec]:
         specs = [TensorSpec(self.spec.embedding, (self.spec.vocab_size, self.spec.hidden_size), MATRIX)]
+        if self.spec.position_table is not None:
+            specs.append(TensorSpec(self.spec.position_table, (self.spec.max_positions, self.spec.hidden_size), MATRIX))
         for layer in self.layers:
             specs += layer.tensor_specs()
         specs += self.final_norm.tensor_specs()
@@ -85,6 +89,8 @@ class DecoderModel:
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         tensors = dict(tensors)
         self.embedding = tensors.pop(self.spec.embedding).contiguous()
+        if self.spec.position_table is not None:
+            self.position_table = tensors.pop(self.spec.position_table).contiguous()
         self.head = tensors.pop(self.spec.head).contiguous() if self.spec.head is not None else self.embedding
         for layer in self.layers:
             layer.bind(tensors)
@@ -152,6 +158,8 @@ class DecoderModel:
         resident: Dict[str, int] = {"embed": 0, "head": 0}
         table = TensorSpec(self.spec.embedding, (self.spec.vocab_size, self.spec.hidden_size), MATRIX)
         resident["embed"] = nbytes(table)
+        if self.spec.position_table is not None:
+            resident["positions"] = nbytes(TensorSpec(self.spec.position_table, (self.spec.max_positions, self.spec.hidden_size), MATRIX))
         if self.spec.head is not None:
             resident["head"] = nbytes(TensorSpec(self.spec.head, (self.spec.vocab_size, self.spec.hidden_size), MATRIX))
         for layer in self.layers:
@@ -161,6 +169,8 @@ class DecoderModel:
         resident["norm"] = resident.get("norm", 0) + sum(nbytes(s) for s in self.final_norm.tensor_specs())
         decode = dict(resident)
         decode["embed"] = resident["embed"] // self.spec.vocab_size * rows
+        if "positions" in decode:
+            decode["positions"] = resident["positions"] // self.spec.max_positions * rows
         if self.spec.head is None:
             decode["head"] = resident["embed"]
         return {"tensor_bytes": sum(resident.values()), "resident": resident, "decode": decode,
@@ -222,7 +232,10 @@ class DecoderModel:
     # ---- forward ---------------------------------------------------------------
     def forward(self, tokens: torch.Tensor, step: StepContext, caches: Dict[int, CacheView]) -> Optional[torch.Tensor]:
         """Runs the step's rows through every scheduled layer; returns float32 logits of the wanted rows."""
-        x = ops.embed(self.embedding, tokens, scale=self.spec.embedding_scale or 1.0)
+        if self.position_table is not None and step.max_position >= self.position_table.shape[0]:
+            raise ValueError(f"position {step.max_position} is beyond the position table of {self.position_table.shape[0]} rows")
+        x = ops.embed(self.embedding, tokens, scale=self.spec.embedding_scale or 1.0,
+                      position_table=self.position_table, positions=step.positions)
         pending = None
         for at, run in enumerate(self.schedule):
             layer = self.layers[run.layer]

@@ -36,8 +36,21 @@ class RmsNorm(Part):
         if isinstance(delta, ops.PreparedRows):
             delta = None                      # the product that made it has added into the stream already
         if isinstance(delta, ops.NormedDelta):
+            behind = delta.norm
+            if isinstance(behind, RmsNorm) and behind.gain.dtype == self.gain.dtype:
+                # the norm behind the last sublayer, the residual sum and this norm in one kernel
+                return ops.add_normed(x, delta.rows, behind.gain, behind.eps, then=(self.gain, self.eps, out_dtype), rows=rows)
             delta = delta.materialize()       # a delta that another kind of norm is still to be applied to
         return ops.add_rmsnorm(x, delta, self.gain, self.eps, out_dtype, rows)
+
+    def apply(self, rows: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        """The norm of float32 rows that are no stream (nothing is added, nothing written back)."""
+        return ops.add_rmsnorm(rows, None, self.gain, self.eps, out_dtype)
+
+    def add_behind(self, x: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: Optional[torch.dtype]):
+        """For a norm that stands behind its sublayer: x += norm(delta) in the float32 stream, and the new rows of
+        the stream come back in ``out_dtype`` (what the next sublayer's products read; None: nothing comes back)."""
+        return ops.add_normed(x, delta, self.gain, self.eps, out_dtype=out_dtype)
 
     def folded(self, out_dtype: torch.dtype):
         """(gain, eps, type) for a product that can leave this norm's operand behind when it adds into the
