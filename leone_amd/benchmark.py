@@ -369,6 +369,31 @@ def pamevik_shape(width: int, layers: int, vocab: int, context: int) -> dict:
             "max_positions": max(4096, context + 64), "layers": [order[i % 4] for i in range(layers)]}
 
 
+def zukinex_shape(width: int, layers: int, vocab: int, context: int) -> dict:
+    """Zukinex at layer sizes that resemble published models of its kind: heads of 128 with four query heads a key
+    head, half of a head rotated, a window of 1,024 with four kept first keys, every other layer reading the keys of
+    the layer before it; the first layer's feed-forward dense (3 x width), the others 32 experts of 3/8 width with
+    four chosen (three identity experts beside them, seven groups of five of which four stay open) and a shared
+    expert of 3/4 width: 2.25 x width of feed-forward a token."""
+    def mixer(kv_from=None):
+        m = {"heads": width // 128, "kv_heads": width // 512, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+             "rot": {"dims": 64, "base": 1000000.0}, "mask": {"size": 1024, "keep_first": 4}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return m
+    routed = {"kind": "moe", "expert": {"ff": 3 * width // 8}, "shared": {"ff": 3 * width // 4},
+              "router": {"experts": 32, "identity": 3, "top": 4, "groups": {"count": 7, "keep": 4}}}
+    listed = []
+    for i in range(layers):
+        listed.append({"type": "attention", "mixer": mixer(i - 1 if i % 2 else None),
+                       "mlp": {"kind": "dense", "ff": 3 * width} if i == 0 else routed})
+    return {"architecture": "Zukinex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "max_positions": max(4096, context + 64), "layers": listed}
+
+
+DESIGN_SHAPES = {"pamevik": pamevik_shape, "zukinex": zukinex_shape}
+
+
 def state_bytes_per_request(model) -> int:
     """Bytes of per-request state a decode step reads and writes back (both ways counted)."""
     total = 0
@@ -382,7 +407,7 @@ def state_bytes_per_request(model) -> int:
 
 
 def run_design(name: str, sizes: List[str], steps: int, warmup: int) -> dict:
-    """Decode and prefill throughput of ``name`` ("pamevik") at DESIGN_SIZES, each beside Qwen3 at the same width,
+    """Decode and prefill throughput of ``name`` (a key of DESIGN_SHAPES) at DESIGN_SIZES, each beside Qwen3 at the same width,
     layers and vocabulary, with a per-operation table of a decode step and of the prompt's step for both."""
     import torch
     from .architectures import config_from_dict
@@ -417,7 +442,7 @@ def run_design(name: str, sizes: List[str], steps: int, warmup: int) -> dict:
     points = {}
     for key in sizes:
         size = DESIGN_SIZES[key]
-        new = measure(pamevik_shape(size["width"], size["layers"], size["vocab"], max(size["context"], size["prompt"])), size)
+        new = measure(DESIGN_SHAPES[name](size["width"], size["layers"], size["vocab"], max(size["context"], size["prompt"])), size)
         beside = measure(dict(QWEN3_8B, num_hidden_layers=size["layers"], hidden_size=size["width"],
                               num_attention_heads=size["width"] // 128, num_key_value_heads=size["width"] // 512,
                               intermediate_size=3 * size["width"], vocab_size=size["vocab"],
@@ -432,7 +457,7 @@ def run_design(name: str, sizes: List[str], steps: int, warmup: int) -> dict:
 
 def main(argv: Optional[List[str]] = None) -> int:
     parser = argparse.ArgumentParser(prog="bench.py")
-    parser.add_argument("--design", choices=["pamevik"],
+    parser.add_argument("--design", choices=sorted(DESIGN_SHAPES),
                         help="instead of the headline figure: this design at a few layer sizes beside Qwen3 at equal size "
                              "(decode and prefill throughput, per-operation times)")
     parser.add_argument("--design-sizes", default="w2048,w4096", help="which of " + ", ".join(sorted(DESIGN_SIZES)))

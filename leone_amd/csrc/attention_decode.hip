@@ -127,7 +127,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                         const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
                         float* __restrict__ part_acc, float* __restrict__ part_ml, bf16_t* __restrict__ out,
                         int q_heads, int kv_heads, int page_shift, float to_log2, int window, int splits,
-                        FromProjection from) {
+                        FromProjection from, int keep_first) {
     constexpr int kD = kD16 * 16;
     constexpr int kSteps = (kD16 + 1) / 2;           // 32-element steps of the q.k product
     extern __shared__ float smem[];                   // [waves][columns][kD] accumulators, then m and l
@@ -149,24 +149,49 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     const int lo = (window > 0 && n - window > 0) ? n - window : 0;      // first key in reach
     const int* table = block_table + static_cast<long>(row_entry[row]) * max_blocks;
     const int t_begin = lo / kTileKeys, t_end = (n + kTileKeys - 1) / kTileKeys;
-    const int per_split = (t_end - t_begin + splits - 1) / splits;
-    const int my_begin = t_begin + split * per_split;
-    const int my_end = my_begin + per_split < t_end ? my_begin + per_split : t_end;
+    // A windowed layer may keep its first keys in sight: keys below `keep` count as in reach wherever they lie.
+    // The tiles that hold such keys and lie wholly before the window's first tile come first in the row's list of
+    // tiles (`kept_tiles` of them), then the window's tiles; a tile of the list is `tile_of(u)`.
+    const int keep = lo > 0 ? (keep_first < lo ? keep_first : lo) : 0;
+    const int kept_all = (keep + kTileKeys - 1) / kTileKeys;
+    const int kept_tiles = kept_all < t_begin ? kept_all : t_begin;
+    const int n_tiles = kept_tiles + t_end - t_begin;
+    auto tile_of = [&](int u) { return u < kept_tiles ? u : t_begin + (u - kept_tiles); };
+    auto in_reach = [&](int key) { return key < n && (key >= lo || key < keep); };
+    const int per_split = (n_tiles + splits - 1) / splits;
+    const int my_begin = split * per_split;                         // places in the row's list of tiles
+    const int my_end = my_begin + per_split < n_tiles ? my_begin + per_split : n_tiles;
 
     // The page ids of this split's keys go to shared memory first: no load of keys or values then
-    // waits on a read of the block table.
+    // waits on a read of the block table.  The window's pages, then those of the kept first keys before them.
     int* pages = reinterpret_cast<int*>(smem + kDecodeWaves * cols * (kD + 2));
-    const int first_page = (my_begin * kTileKeys) >> page_shift;
-    {
-        const int last_key = (my_end * kTileKeys < n ? my_end * kTileKeys : n) - 1;
-        const int n_pages = my_begin < my_end ? (last_key >> page_shift) - first_page + 1 : 0;
-        for (int i = threadIdx.x; i < n_pages; i += kDecodeThreads) pages[i] = table[first_page + i];
+    const int win_begin = (my_begin > kept_tiles ? my_begin : kept_tiles) - kept_tiles + t_begin;   // tiles of the window in this split
+    const int win_end = my_end - kept_tiles + t_begin;
+    const bool has_window = my_end > kept_tiles && my_begin < my_end;
+    const int first_page = has_window ? (win_begin * kTileKeys) >> page_shift : 0x3fffffff;
+    int n_win_pages = 0;
+    if (has_window) {
+        const int last_key = (win_end * kTileKeys < n ? win_end * kTileKeys : n) - 1;
+        n_win_pages = (last_key >> page_shift) - first_page + 1;
+        for (int i = threadIdx.x; i < n_win_pages; i += kDecodeThreads) pages[i] = table[first_page + i];
     }
+    const int kept_first_page = (my_begin * kTileKeys) >> page_shift;
+    if (my_begin < kept_tiles && my_begin < my_end) {
+        const int last_tile = my_end < kept_tiles ? my_end : kept_tiles;
+        int last_page = (last_tile * kTileKeys - 1) >> page_shift;
+        if (last_page >= first_page) last_page = first_page - 1;        // that page is among the window's
+        for (int i = kept_first_page + threadIdx.x; i <= last_page; i += kDecodeThreads)
+            pages[n_win_pages + i - kept_first_page] = table[i];
+    }
+    auto page_at = [&](int key) {
+        const int b = key >> page_shift;
+        return b >= first_page ? pages[b - first_page] : pages[n_win_pages + b - kept_first_page];
+    };
     if constexpr (kFused) {
         // The workgroup whose keys end with the row's own position makes that position's key and value and
         // writes them into the cache; its waves read them from there after the barrier.  (With more than 16
         // query heads a kv head several workgroups do, each for itself: the same bytes.)
-        if (from.k_out != nullptr && my_begin < my_end && my_end == t_end) {
+        if (from.k_out != nullptr && my_begin < my_end && my_end == n_tiles) {
             const long width = static_cast<long>(q_heads + 2 * kv_heads) * kD;
             const int pos = n - 1;
             const int page = table[pos >> page_shift];
@@ -258,15 +283,15 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     struct Tile {
         bf16x8 xa[kSteps], xb[kSteps], xv[kD16];
     };
-    auto issue = [&](int t, bool exists, Tile& r) {
-        const int key0 = t * kTileKeys;
+    auto issue = [&](int u, bool exists, Tile& r) {
+        const int key0 = (exists ? tile_of(u) : 0) * kTileKeys;
         // A-operand row c of half a is key 8*(c/4) + c%4, of half b four keys further
         const int ka = key0 + 8 * (c >> 2) + (c & 3);
         const int run0 = key0 + 8 * g;                   // this lane's eight keys for the second product
-        const bool near = exists && ka + 4 >= lo && ka < n;   // ka or kb = ka + 4 in reach: they share a page (pages hold multiples of 8 keys)
-        const bool any = exists && run0 < n && run0 + 8 > lo;
-        const int page_k = near ? pages[(ka >> page_shift) - first_page] : -1;
-        const int page_v = any ? pages[(run0 >> page_shift) - first_page] : -1;
+        const bool near = exists && ka < n && (ka + 4 >= lo || ka < keep);   // ka or kb = ka + 4 in reach: they share a page (pages hold multiples of 8 keys)
+        const bool any = exists && run0 < n && (run0 + 8 > lo || run0 < keep);
+        const int page_k = near ? page_at(ka) : -1;
+        const int page_v = any ? page_at(run0) : -1;
         const bf16_t* pk = page_k < 0 ? k_pool
                                       : k_pool + (static_cast<long>(page_k) * kv_heads + kvh) * page_tokens * kD + (ka & page_mask) * 8;
         const bf16_t* pv = page_v < 0 ? v_pool
@@ -357,18 +382,18 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
 #pragma unroll
     for (int dt = 0; dt < kD16; ++dt) acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    auto finish = [&](int t, Tile& r) {
-        const int key0 = t * kTileKeys;
-        const bool full = key0 >= lo && key0 + kTileKeys <= n;      // the same for the whole wave
+    auto finish = [&](int u, Tile& r) {
+        const int key0 = tile_of(u) * kTileKeys;
+        const bool full = (key0 >= lo || key0 + kTileKeys <= keep) && key0 + kTileKeys <= n;      // the same for the whole wave
         const int ka = key0 + 8 * (c >> 2) + (c & 3);
         const int kb = ka + 4;
         const int run0 = key0 + 8 * g;
-        bool va = ka >= lo && ka < n, vb = kb >= lo && kb < n, any = run0 < n && run0 + 8 > lo;
-        if ((va || vb) && pages[(ka >> page_shift) - first_page] < 0) {
+        bool va = in_reach(ka), vb = in_reach(kb), any = run0 < n && (run0 + 8 > lo || run0 < keep);
+        if ((va || vb) && page_at(ka) < 0) {
             unmapped = true;                              // never read outside the pool; the result is poisoned below
             va = vb = false;
         }
-        if (any && pages[(run0 >> page_shift) - first_page] < 0) {
+        if (any && page_at(run0) < 0) {
             unmapped = true;
             any = false;
         }
@@ -380,7 +405,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                 if (!(va && in_head)) r.xa[s] = zero8();
                 if (!(vb && in_head)) r.xb[s] = zero8();
             }
-            const bool whole = run0 >= lo && run0 + 8 <= n;
+            const bool whole = (run0 >= lo || run0 + 8 <= keep) && run0 + 8 <= n;
 #pragma unroll
             for (int dt = 0; dt < kD16; ++dt) {
                 if (!any) {
@@ -393,8 +418,8 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                     for (int i = 0; i < 4; ++i) {
                         const int e0 = run0 + 2 * i, e1 = e0 + 1;
                         unsigned mask = 0u;
-                        if (e0 >= lo && e0 < n) mask |= 0x0000ffffu;
-                        if (e1 >= lo && e1 < n) mask |= 0xffff0000u;
+                        if (in_reach(e0)) mask |= 0x0000ffffu;
+                        if (in_reach(e1)) mask |= 0xffff0000u;
                         w[i] &= mask;
                     }
                     r.xv[dt] = __builtin_bit_cast(bf16x8, raw);
@@ -416,7 +441,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         for (int j = 0; j < 8; ++j) {
             const int key = run0 + j;
             const float raw = j < 4 ? sa[j & 3] : sb[j & 3];
-            sc[j] = (full || (key >= lo && key < n)) ? raw * to_log2 : -INFINITY;
+            sc[j] = (full || in_reach(key)) ? raw * to_log2 : -INFINITY;
             tile_max = fmaxf(tile_max, sc[j]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
@@ -553,7 +578,7 @@ template <int kD16>
 static void launch_decode(const void* q, const void* k_pool, const void* v_pool, const int* positions,
                           const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
                           float* part_ml, void* out, int rows, int q_heads, int kv_heads, int page_shift, float scale,
-                          int window, int splits, const FromProjection* from, hipStream_t stream) {
+                          int window, int splits, const FromProjection* from, int keep_first, hipStream_t stream) {
     const int group = q_heads / kv_heads;
     dim3 grid(rows, kv_heads * ((group + 15) / 16), splits);
     const size_t smem = decode_smem_bytes(kD16 * 16, group, max_blocks);
@@ -563,20 +588,22 @@ static void launch_decode(const void* q, const void* k_pool, const void* v_pool,
             attention_decode_kernel<kD16, true><<<grid, kDecodeThreads, smem, stream>>>(
                 nullptr, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), positions, row_entry,
                 block_table, max_blocks, part_acc, part_ml, static_cast<bf16_t*>(out), q_heads, kv_heads, page_shift,
-                to_log2, window, splits, *from);
+                to_log2, window, splits, *from, keep_first);
             return;
         }
     }
     attention_decode_kernel<kD16, false><<<grid, kDecodeThreads, smem, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
         positions, row_entry, block_table, max_blocks, part_acc, part_ml, static_cast<bf16_t*>(out), q_heads, kv_heads,
-        page_shift, to_log2, window, splits, FromProjection{});
+        page_shift, to_log2, window, splits, FromProjection{}, keep_first);
 }
 
 static int decode_checked(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
                           const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
                           float* part_ml, int rows, int q_heads, int kv_heads, int head_dim, int page_tokens,
-                          float scale, int window, int splits, const FromProjection* from, hipStream_t stream) {
+                          float scale, int window, int splits, const FromProjection* from, int keep_first,
+                          hipStream_t stream) {
+    LEONE_REQUIRE(keep_first >= 0, "attention_decode: keep_first %d must not be negative", keep_first);
     LEONE_REQUIRE((q || from) && out && k_pool && v_pool && positions && row_entry && block_table,
                   "attention_decode: null pointer");
     LEONE_REQUIRE(splits == 1 || (part_acc && part_ml), "attention_decode: %d splits need the workspace", splits);
@@ -599,7 +626,7 @@ static int decode_checked(const void* q, void* out, const void* k_pool, const vo
 #define LEONE_DECODE_CASE(N)                                                                                      \
     case N:                                                                                                       \
         launch_decode<N>(q, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml,     \
-                         out, rows, q_heads, kv_heads, page_shift, scale, window, splits, from, stream);          \
+                         out, rows, q_heads, kv_heads, page_shift, scale, window, splits, from, keep_first, stream); \
         break;
     switch (head_dim / 16) {
         LEONE_DECODE_CASE(1) LEONE_DECODE_CASE(2) LEONE_DECODE_CASE(3) LEONE_DECODE_CASE(4)
@@ -631,7 +658,17 @@ extern "C" int leone_attention_decode(const void* q, void* out, const void* k_po
                                       int kv_heads, int head_dim, int page_tokens, float scale, int window,
                                       int splits, hipStream_t stream) {
     return decode_checked(q, out, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml, rows,
-                          q_heads, kv_heads, head_dim, page_tokens, scale, window, splits, nullptr, stream);
+                          q_heads, kv_heads, head_dim, page_tokens, scale, window, splits, nullptr, 0, stream);
+}
+
+// The same with the keys at positions below keep_first kept in sight of a windowed layer.
+extern "C" int leone_attention_decode_kept(const void* q, void* out, const void* k_pool, const void* v_pool,
+                                           const int* positions, const int* row_entry, const int* block_table,
+                                           int max_blocks, float* part_acc, float* part_ml, int rows, int q_heads,
+                                           int kv_heads, int head_dim, int page_tokens, float scale, int window,
+                                           int splits, int keep_first, hipStream_t stream) {
+    return decode_checked(q, out, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml, rows,
+                          q_heads, kv_heads, head_dim, page_tokens, scale, window, splits, nullptr, keep_first, stream);
 }
 
 // The same for a step in which every row is another request, taking the fused q/k/v projection instead of
@@ -667,5 +704,5 @@ extern "C" int leone_attention_decode_projected(const void* qkv, int qkv_dtype, 
                         write_cache ? static_cast<bf16_t*>(k_pool) : nullptr,
                         write_cache ? static_cast<bf16_t*>(v_pool) : nullptr};
     return decode_checked(nullptr, out, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml,
-                          rows, q_heads, kv_heads, head_dim, page_tokens, scale, window, splits, &from, stream);
+                          rows, q_heads, kv_heads, head_dim, page_tokens, scale, window, splits, &from, 0, stream);
 }

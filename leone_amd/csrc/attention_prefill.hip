@@ -72,7 +72,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                          const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
                          const int* __restrict__ tiles, int n_groups, const int* __restrict__ block_table,
                          int max_blocks, int q_heads, int kv_heads, int page_shift, float scale, int window,
-                         float* __restrict__ part_acc, float* __restrict__ part_ml, int splits) {
+                         float* __restrict__ part_acc, float* __restrict__ part_ml, int splits, int keep_first) {
     constexpr int kD = kD16 * 16;
     constexpr int kRuns = kD / 8;                      // 16-byte runs of one key
     constexpr int kDT = (kD + 31) / 32;                // 32-row tiles of the second product's result
@@ -147,6 +147,15 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     const int* table = block_table + static_cast<long>(entry) * max_blocks;
     for (int i = tid; i < n_pages; i += kPrefillThreads) pages[i] = table[first_page + i];
     __syncthreads();
+    // A windowed layer may keep its first keys in sight: keys below `keep` are read wherever they lie (the host
+    // asks for them only with one range of keys).  Their pages, where they lie before the window's, are read
+    // from the block table itself.
+    const int keep = (window > 0 && splits == 1) ? keep_first : 0;
+    auto page_at = [&](int key) {
+        const int b = key >> page_shift;
+        return b >= first_page ? pages[b - first_page] : table[b];
+    };
+    auto in_range = [&](int key) { return key < group_hi && (key >= group_lo || key < keep); };
 
     // The Q^T operand and the row's own position.
     const bool row_ok = j < wave_rows;
@@ -210,8 +219,8 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             if (kKeyRuns % kPrefillThreads != 0 && idx >= kKeyRuns) continue;
             {
                 const int run = idx / kStageKeys, key = key_base + idx % kStageKeys;
-                if (key >= group_lo && key < group_hi) {
-                    const int page = pages[(key >> page_shift) - first_page];
+                if (in_range(key)) {
+                    const int page = page_at(key);
                     if (page < 0) {
                         unmapped_seen = 1;
                     } else {
@@ -222,8 +231,8 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             }
             {
                 const int tg = idx / kD, d = idx % kD, key = key_base + 8 * tg;
-                if (key < group_hi && key + 8 > group_lo) {
-                    const int page = pages[(key >> page_shift) - first_page];
+                if (key < group_hi && (key + 8 > group_lo || key < keep)) {
+                    const int page = page_at(key);
                     if (page < 0) {
                         unmapped_seen = 1;
                     } else {
@@ -235,8 +244,8 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                             for (int h = 0; h < 4; ++h) {
                                 const int e0 = key + 2 * h, e1 = e0 + 1;
                                 unsigned mask = 0u;
-                                if (e0 >= group_lo && e0 < group_hi) mask |= 0x0000ffffu;
-                                if (e1 >= group_lo && e1 < group_hi) mask |= 0xffff0000u;
+                                if (in_range(e0)) mask |= 0x0000ffffu;
+                                if (in_range(e1)) mask |= 0xffff0000u;
                                 w[h] &= mask;
                             }
                         }
@@ -319,7 +328,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int key = key0 + 8 * h + (v & 7) + 16 * (v >> 3);
-                sc[v] = (key <= row_pos && key >= p_lo) ? sc[v] : -INFINITY;
+                sc[v] = (key <= row_pos && (key >= p_lo || key < keep)) ? sc[v] : -INFINITY;
             }
         }
         float top = sc[0];
@@ -361,13 +370,19 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     };
 
     const int t_begin = group_lo / kStageKeys, t_end = (group_hi + kStageKeys - 1) / kStageKeys;
-    if (!fetch(t_begin, shared)) deposit(shared);
+    // The stages that hold kept first keys and lie wholly before the window's first stage come first.
+    const int kept_keys = keep < group_lo ? keep : group_lo;
+    const int kept_all = (kept_keys + kStageKeys - 1) / kStageKeys;
+    const int kept_stages = kept_all < t_begin ? kept_all : t_begin;
+    const int n_stages = kept_stages + t_end - t_begin;
+    auto stage_of = [&](int u) { return u < kept_stages ? u : t_begin + (u - kept_stages); };
+    if (!fetch(stage_of(0), shared)) deposit(shared);
     arrived();
     __syncthreads();
     // One round: start bringing the next stage to `writing`, work on the present one in `reading`.  The two
     // are told apart for the compiler (they never overlap), so that it does not wait for the runs on their way
     // to `writing` before it reads `reading`.
-    auto round = [&](const uint4* __restrict__ reading, uint4* __restrict__ writing, int t, bool more) {
+    auto round = [&](const uint4* __restrict__ reading, uint4* __restrict__ writing, int t, int t_next, bool more) {
         // `writing` was last read before the barrier that ended the round before: it is free.  The next
         // stage is sent for between the two halves (measured: better than before the first half, where its
         // arrival in shared memory gets in the way of the reads of both halves).
@@ -375,15 +390,15 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
         for (int half = 0; half < kStageKeys / kKeysPerPass; ++half) {
             const int key0 = t * kStageKeys + half * kKeysPerPass;
-            if (half == kStageKeys / kKeysPerPass - 1) direct = more && fetch(t + 1, writing);
-            if (key0 >= key_hi || key0 + kKeysPerPass <= key_lo) continue;      // nothing of it for this wave
+            if (half == kStageKeys / kKeysPerPass - 1) direct = more && fetch(t_next, writing);
+            if (key0 >= key_hi || (key0 + kKeysPerPass <= key_lo && key0 >= keep)) continue;      // nothing of it for this wave
             pass(reading, key0, half, key0 >= full_lo && key0 + kKeysPerPass <= full_hi);
         }
         if (more && !direct) deposit(writing);
     };
     int cur = 0;
-    for (int t = t_begin; t < t_end; ++t) {
-        round(shared + cur * kStageRuns, shared + (cur ^ 1) * kStageRuns, t, t + 1 < t_end);
+    for (int u = 0; u < n_stages; ++u) {
+        round(shared + cur * kStageRuns, shared + (cur ^ 1) * kStageRuns, stage_of(u), stage_of(u + 1), u + 1 < n_stages);
         arrived();
         __syncthreads();
         cur ^= 1;
@@ -480,7 +495,7 @@ template <int kD16>
 static int launch_prefill(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
                           const int* tiles, int n_groups, const int* block_table, int max_blocks, int q_heads,
                           int kv_heads, int page_shift, float scale, int window, float* part_acc, float* part_ml,
-                          int splits, hipStream_t stream) {
+                          int splits, int keep_first, hipStream_t stream) {
     const size_t shared = 2 * static_cast<size_t>(stage_runs(16 * kD16)) * sizeof(uint4) + static_cast<size_t>(max_blocks) * sizeof(int);
     static size_t allowed = 48 * 1024;                 // what a kernel may use without asking
     if (shared > allowed) {
@@ -495,7 +510,7 @@ static int launch_prefill(const void* q, void* out, const void* k_pool, const vo
     attention_prefill_kernel<kD16><<<dim3(n_groups * q_heads, splits), kPrefillThreads, shared, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), positions, tiles, n_groups, block_table, max_blocks, q_heads, kv_heads,
-        page_shift, scale, window, part_acc, part_ml, splits);
+        page_shift, scale, window, part_acc, part_ml, splits, keep_first);
     return 0;
 }
 
@@ -512,11 +527,29 @@ extern "C" int leone_attention_prefill_max_splits() { return kMaxPrefillSplits; 
 // splits > 1 cuts every workgroup's keys into that many ranges and needs the workspace: part_acc of
 // rows * q_heads * splits * head_dim floats and part_ml of rows * q_heads * splits * 2, `rows` being one
 // more than the last row any tile names; with splits == 1 both may be null.
+extern "C" int leone_attention_prefill_kept(const void* q, void* out, const void* k_pool, const void* v_pool,
+                                            const int* positions, const int* tiles, int n_groups, const int* block_table,
+                                            int max_blocks, int q_heads, int kv_heads, int head_dim, int page_tokens,
+                                            float scale, int window, float* part_acc, float* part_ml, int splits,
+                                            int keep_first, hipStream_t stream);
+
 extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_pool, const void* v_pool,
                                        const int* positions, const int* tiles, int n_groups, const int* block_table,
                                        int max_blocks, int q_heads, int kv_heads, int head_dim, int page_tokens,
                                        float scale, int window, float* part_acc, float* part_ml, int splits,
                                        hipStream_t stream) {
+    return leone_attention_prefill_kept(q, out, k_pool, v_pool, positions, tiles, n_groups, block_table, max_blocks, q_heads,
+                                        kv_heads, head_dim, page_tokens, scale, window, part_acc, part_ml, splits, 0, stream);
+}
+
+// The same with the keys at positions below keep_first kept in sight of a windowed layer (one range of keys only).
+extern "C" int leone_attention_prefill_kept(const void* q, void* out, const void* k_pool, const void* v_pool,
+                                            const int* positions, const int* tiles, int n_groups, const int* block_table,
+                                            int max_blocks, int q_heads, int kv_heads, int head_dim, int page_tokens,
+                                            float scale, int window, float* part_acc, float* part_ml, int splits,
+                                            int keep_first, hipStream_t stream) {
+    LEONE_REQUIRE(keep_first >= 0 && (keep_first == 0 || window == 0 || splits == 1),
+                  "attention_prefill: kept first keys (%d) beside a window come with one range of keys, not %d", keep_first, splits);
     LEONE_REQUIRE(q && out && k_pool && v_pool && positions && tiles && block_table, "attention_prefill: null pointer");
     LEONE_REQUIRE(n_groups > 0 && q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
                   "attention_prefill: %d tile groups, %d query heads over %d kv heads", n_groups, q_heads, kv_heads);
@@ -540,7 +573,7 @@ extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_p
     case N:                                                                                                        \
         status = launch_prefill<N>(q, out, k_pool, v_pool, positions, tiles, n_groups, block_table, max_blocks,    \
                                    q_heads, kv_heads, page_shift, scale, window, part_acc, part_ml, splits,        \
-                                   stream);                                                                        \
+                                   keep_first, stream);                                                            \
         break;
     switch (head_dim / 16) {
         LEONE_PREFILL_CASE(1) LEONE_PREFILL_CASE(2) LEONE_PREFILL_CASE(3) LEONE_PREFILL_CASE(4)

@@ -272,6 +272,16 @@ int leone_attention_rows_kept(const void* q, void* out, const void* k_pool, cons
                               int rows, int q_heads, int kv_heads, int head_dim, int v_dim, int page_tokens,
                               float scale, int window, const float* gate, long gate_stride, int keep_first,
                               int gate_each, hipStream_t stream);
+// leone_attention_decode with the keys at positions below keep_first kept in sight of a windowed layer.
+int leone_attention_decode_kept(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
+                                const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
+                                float* part_ml, int rows, int q_heads, int kv_heads, int head_dim, int page_tokens,
+                                float scale, int window, int splits, int keep_first, hipStream_t stream);
+// leone_attention_prefill with the keys at positions below keep_first kept in sight of a windowed layer (splits 1).
+int leone_attention_prefill_kept(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
+                                 const int* tiles, int n_groups, const int* block_table, int max_blocks, int q_heads,
+                                 int kv_heads, int head_dim, int page_tokens, float scale, int window, float* part_acc,
+                                 float* part_ml, int splits, int keep_first, hipStream_t stream);
 // Router: chosen int32 [rows, top], weight float32 [rows, top] from logits float32 [rows, total] (see routed.hip).
 int leone_route_max_outputs();
 int leone_route_topk(const float* logits, const void* correction, int correction_dtype, int* chosen, float* weight,

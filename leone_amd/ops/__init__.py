@@ -351,26 +351,28 @@ def choose_splits(rows: int, kv_heads: int, group: int, max_context: int, units:
 def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
                      row_entry: torch.Tensor, block_table: torch.Tensor, q_heads: int, scale: float,
                      window: int = 0, max_context: int = 1, splits: Optional[int] = None,
-                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Split-KV attention on the matrix cores (bfloat16).  ``max_context`` only steers the number of splits."""
+                     out: Optional[torch.Tensor] = None, keep_first: int = 0) -> torch.Tensor:
+    """Split-KV attention on the matrix cores (bfloat16).  ``max_context`` only steers the number of splits.
+    ``keep_first``: keys at positions below it stay in sight of a windowed layer."""
     rows = q.shape[0]
     pages, kv_heads, page_tokens, head_dim = cache_dims(k_pool, v_pool)
     if q.shape[1] != q_heads * head_dim:
         raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
     if splits is None:
-        splits = choose_splits(rows, kv_heads, q_heads // kv_heads, max_context, compute_units(q.device))
+        reach = min(max_context, window + keep_first + 32) if window else max_context     # keys a row can see at most
+        splits = choose_splits(rows, kv_heads, q_heads // kv_heads, reach, compute_units(q.device))
     if out is None:
         out = torch.empty_like(q)
     part_acc = part_ml = None
     if splits > 1:
         part_acc = torch.empty((rows * q_heads * splits * head_dim,), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((rows * q_heads * splits * 2,), dtype=torch.float32, device=q.device)
-    call("leone_attention_decode", _dev(q, "attention q", torch.bfloat16),
+    call("leone_attention_decode_kept", _dev(q, "attention q", torch.bfloat16),
          _dev(out, "attention out", torch.bfloat16, q.shape), _dev(k_pool, "k pool", torch.bfloat16),
          _dev(v_pool, "v pool", torch.bfloat16), _dev(positions, "positions", torch.int32, (rows,)),
          _dev(row_entry, "row map", torch.int32, (rows,)), _dev(block_table, "block table", torch.int32),
          block_table.shape[1], _dev(part_acc, "partials"), _dev(part_ml, "partial sums"), rows, q_heads, kv_heads,
-         head_dim, page_tokens, float(scale), int(window), int(splits), _stream())
+         head_dim, page_tokens, float(scale), int(window), int(splits), int(keep_first) if window else 0, _stream())
     return out
 
 
@@ -459,14 +461,15 @@ def choose_prefill_splits(groups: int, q_heads: int, mean_keys: int, window: int
 def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                       positions: torch.Tensor, tiles: torch.Tensor, block_table: torch.Tensor, q_heads: int,
                       scale: float, window: int = 0, mean_keys: int = 1, splits: Optional[int] = None,
-                      covered_rows: Optional[int] = None) -> torch.Tensor:
+                      covered_rows: Optional[int] = None, keep_first: int = 0) -> torch.Tensor:
     """Attention for the rows that ``tiles`` covers; writes into ``out``.
 
     ``tiles`` is int32 [n, 3]: (entry, first row, rows) with at most PREFILL_TILE_ROWS consecutive rows of one
     request each, PREFILL_GROUP_TILES to a group, all tiles of a group of the same entry, unused places with
     0 rows (``prefill_tiles`` builds such a list).  ``mean_keys`` (keys a row sees on average) only steers
     the number of key ranges (``splits``); ``covered_rows``: one more than the last row a tile names, if the
-    caller knows it."""
+    caller knows it.  ``keep_first``: keys at positions below it stay in sight of a windowed layer (the keys are
+    then walked as one range)."""
     if (library().leone_attention_prefill_tile_rows() != PREFILL_TILE_ROWS
             or library().leone_attention_prefill_group_tiles() != PREFILL_GROUP_TILES
             or library().leone_attention_prefill_max_splits() != PREFILL_MAX_SPLITS):
@@ -478,6 +481,9 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, 
     if tiles.dim() != 2 or tiles.shape[1] != 3 or tiles.shape[0] % PREFILL_GROUP_TILES:
         raise KernelError(f"attention_prefill: tiles must be int32 [n, 3] with n a multiple of {PREFILL_GROUP_TILES}")
     groups = tiles.shape[0] // PREFILL_GROUP_TILES
+    keep_first = int(keep_first) if window else 0
+    if keep_first:
+        splits = 1
     if splits is None:
         splits = choose_prefill_splits(groups, q_heads, mean_keys, window, compute_units(q.device))
     part_acc = part_ml = None
@@ -487,12 +493,12 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, 
             raise KernelError(f"attention_prefill: {covered} covered rows of {rows}")
         part_acc = torch.empty((covered * q_heads * splits * head_dim,), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((covered * q_heads * splits * 2,), dtype=torch.float32, device=q.device)
-    call("leone_attention_prefill", _dev(q, "attention q", torch.bfloat16),
+    call("leone_attention_prefill_kept", _dev(q, "attention q", torch.bfloat16),
          _dev(out, "attention out", torch.bfloat16, q.shape), _dev(k_pool, "k pool", torch.bfloat16),
          _dev(v_pool, "v pool", torch.bfloat16), _dev(positions, "positions", torch.int32, (rows,)),
          _dev(tiles, "tiles", torch.int32), groups, _dev(block_table, "block table", torch.int32),
          block_table.shape[1], q_heads, kv_heads, head_dim, page_tokens, float(scale), int(window),
-         _dev(part_acc, "partials"), _dev(part_ml, "partial sums"), int(splits), _stream())
+         _dev(part_acc, "partials"), _dev(part_ml, "partial sums"), int(splits), keep_first, _stream())
     return out
 
 

@@ -73,6 +73,10 @@ _PROTOTYPES = {
     "leone_add_normed": [P, P, c_int, ctypes.c_long, P, c_int, c_float, P, c_int, P, c_int, c_float, P, c_int, c_int, P],
     "leone_attention_rows_kept": [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                   c_int, P, ctypes.c_long, c_int, c_int, P],
+    "leone_attention_decode_kept": [P, P, P, P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                    c_int, c_int, P],
+    "leone_attention_prefill_kept": [P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P, P,
+                                     c_int, c_int, P],
     "leone_route_topk": [P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "leone_moe_plan": [P, c_int, c_int, P, P, c_int, P],
     "leone_moe_product": [P, P, P, P, c_int, c_int, P, P, c_int, c_int, c_int, c_int, c_int, P],

@@ -51,6 +51,8 @@ OPERATIONS = {
     "leone_glu": "swiglu",
     "leone_add_normed": "norm",
     "leone_attention_rows_kept": "attention",
+    "leone_attention_decode_kept": "attention",
+    "leone_attention_prefill_kept": "attention",
     "leone_route_topk": "router",
     "leone_moe_plan": "router",
     "leone_moe_product": "experts",

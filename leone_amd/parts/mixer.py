@@ -179,9 +179,8 @@ class GqaAttention(Part):
                 "prompt": "flash" if ops.prefill_attention_supported(dtype, self.head_dim, page_tokens, max_blocks) else "split_kv"}
 
     def _rows_only(self) -> bool:
-        """What the matrix-core kernels are not built for: values of another size than the keys, kept first keys
-        beside a window, a gate for every element."""
-        return self.value_dim != self.head_dim or bool(self.window and self.keep_first) or self.gate_each
+        """What the matrix-core kernels are not built for: values of another size than the keys."""
+        return self.value_dim != self.head_dim
 
     def _attend(self, q: torch.Tensor, step: StepContext, cache: KvCacheView, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Long prompt portions through the prompt kernel, the other rows through the split-KV kernel; the
@@ -202,10 +201,15 @@ class GqaAttention(Part):
                 and ops.prefill_attention_supported(q.dtype, self.head_dim, cache.page_tokens, max_blocks)):
             ops.attention_prefill(q, out, cache.k_pool, cache.v_pool, step.positions, tiled.tiles,
                                   cache.block_table, self.q_heads, self.scale, window,
-                                  mean_keys=tiled.mean_keys or step.max_position + 1, covered_rows=tiled.rows)
+                                  mean_keys=tiled.mean_keys or step.max_position + 1, covered_rows=tiled.rows,
+                                  keep_first=self.keep_first)
             first = tiled.rows
         if first < step.rows:
             ops.attention_decode(q[first:], cache.k_pool, cache.v_pool, step.positions[first:],
                                  step.row_entry[first:], cache.block_table, self.q_heads, self.scale, window,
-                                 max_context=step.max_position + 1, out=out[first:])
-        return out if gate is None else ops.head_gate(out, gate, self.q_heads, self.value_dim)
+                                 max_context=step.max_position + 1, out=out[first:], keep_first=self.keep_first)
+        if gate is None:
+            return out
+        # a gate for every element is a gate a head of one element
+        return ops.head_gate(out, gate, self.q_heads * self.value_dim, 1) if self.gate_each else \
+            ops.head_gate(out, gate, self.q_heads, self.value_dim)

@@ -64,20 +64,22 @@ def test_a_serving_scenario_with_one_layer(name):
     assert len(record["config"]) <= 20
 
 
-def test_another_design_beside_its_closest_relative(capsys):
-    """``--design pamevik``: one line with the design's decode and prompt figures and Qwen3's at equal width, depth
+@pytest.mark.parametrize("design,operations", [("pamevik", {"outer scan", "delta scan", "layer norm"}),
+                                               ("zukinex", {"router", "experts", "attention", "norm"})])
+def test_another_design_beside_its_closest_relative(capsys, design, operations):
+    """``--design NAME``: one line with the design's decode and prompt figures and Qwen3's at equal width, depth
     and vocabulary beside them, each with a per-operation table; the headline workload is not run."""
     from leone_amd import benchmark
-    assert benchmark.main(["--design", "pamevik", "--design-sizes", "w512", "--steps", "4", "--warmup", "1"]) == 0
+    assert benchmark.main(["--design", design, "--design-sizes", "w512", "--steps", "4", "--warmup", "1"]) == 0
     lines = [line for line in capsys.readouterr().out.splitlines() if line.strip()]
     assert len(lines) == 1
     record = json.loads(lines[0])
-    assert record["n_gpus"] == 1 and record["steps"] == 4 and record["config"] == {"model": "pamevik", "sizes": ["w512"]}
+    assert record["n_gpus"] == 1 and record["steps"] == 4 and record["config"] == {"model": design, "sizes": ["w512"]}
     point = record["points"]["w512"]
-    for name in ("pamevik", "qwen3"):
+    for name in (design, "qwen3"):
         side = point[name]
         assert side["decode_tok_s"] > 0 and side["prefill_tok_s"] > 0 and side["decode_gb_per_step"] > 0
         assert abs(side["decode_tok_s"] - 2 / side["decode_ms_per_step"] * 1e3) / side["decode_tok_s"] < 1e-2
         assert side["decode_operations_us"] and side["prefill_operations_us"]
-    assert record["value"] == point["pamevik"]["decode_tok_s"]
-    assert {"outer scan", "delta scan", "layer norm"} <= set(point["pamevik"]["decode_operations_us"])
+    assert record["value"] == point[design]["decode_tok_s"]
+    assert operations <= set(point[design]["decode_operations_us"])

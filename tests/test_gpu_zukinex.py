@@ -405,6 +405,49 @@ def test_planted_keys_far_away_and_at_every_edge(dtype, window, keep_first):
         assert (hit < 0.25) == bool(see[i, j]), f"position {i}, key {j}: in sight {bool(see[i, j])}, distance {hit:.3f}"
 
 
+@pytest.mark.parametrize("page_tokens", [16, 64])
+@pytest.mark.parametrize("window,keep_first", [(40, 5), (64, 3), (100, 70), (33, 0), (0, 0), (7, 20), (150, 40), (130, 129)])
+def test_matrix_core_attention_with_kept_first_keys(window, keep_first, page_tokens):
+    """The prompt kernel (a portion of 420 rows that continues a request of 100) and the split-KV kernel (the same
+    rows one by one, and cut into several parts) with planted keys: for every row a key at one of the edges (just
+    inside and outside the window, the last kept key and the first that is not, the first key, the row's own, one
+    far back).  Kept keys lie in tiles and stages of their own, before the window's; with 70 and 129 of them they
+    take several."""
+    from leone_amd import ops
+    n, first, heads, q_heads, dim = 520, 100, 2, 4, 32
+    k, v = planted(n, heads, dim, dim, 11 + window)
+    kd, vd = k.bfloat16().float(), v.bfloat16().float()
+    k_pool, v_pool, table = paged(k, v, page_tokens, torch.bfloat16, 9)
+    positions = list(range(first, n))
+    q = torch.zeros(len(positions), q_heads, dim)
+    targets = []
+    for r, i in enumerate(positions):
+        kinds = [i, i - 1, 0, keep_first - 1, keep_first, i // 2, i - window, i - window + 1, i - window - 1, 63, 64]
+        j = kinds[r % len(kinds)] if window else kinds[r % 6]
+        j = min(max(j, 0), i)
+        targets.append(j)
+        for head in range(q_heads):
+            key = kd[j, head // 2]
+            q[r, head] = key / (key @ key) * 60.0
+    want = attend_plainly(q.bfloat16().float(), kd, vd, positions, 1.0, window, keep_first, 2)
+    flat_q = q.reshape(len(positions), -1).bfloat16().to(DEV)
+    rows_at = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    entry = torch.zeros(len(positions), dtype=torch.int32, device=DEV)
+    out = torch.full_like(flat_q, float("nan"))
+    tiles = ops.prefill_tiles([(0, 0, len(positions))]).to(DEV)
+    ops.attention_prefill(flat_q, out, k_pool, v_pool, rows_at, tiles, table, q_heads, 1.0, window, mean_keys=300,
+                          keep_first=keep_first)
+    close(out.float().view(len(positions), q_heads, dim), want, 1.5e-2, "prompt kernel")
+    for splits in (None, 1, 3):
+        one = ops.attention_decode(flat_q, k_pool, v_pool, rows_at, entry, table, q_heads, 1.0, window, max_context=n,
+                                   splits=splits, keep_first=keep_first)
+        close(one.float().view(len(positions), q_heads, dim), want, 1.5e-2, f"split-KV kernel, splits {splits}")
+    see = plain.visible(n, window or None, keep_first)
+    for r, (i, j) in enumerate(zip(positions, targets)):
+        hit = float((out[r].float().cpu().view(q_heads, dim)[0] - vd[j, 0]).abs().max())
+        assert (hit < 0.25) == bool(see[i, j]), f"position {i}, key {j}: in sight {bool(see[i, j])}, distance {hit:.3f}"
+
+
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 def test_attention_layers_alone_with_a_reader_of_the_owners_keys(dtype_name):
     """Two attention parts on one cache slot, the owner of the keys and a reader with a wider mask, fed two
