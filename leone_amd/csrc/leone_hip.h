@@ -286,14 +286,15 @@ int leone_attention_prefill_kept(const void* q, void* out, const void* k_pool, c
 int leone_route_max_outputs();
 int leone_route_topk(const float* logits, const void* correction, int correction_dtype, int* chosen, float* weight,
                      int rows, int total, int top, int group_count, int group_keep, hipStream_t stream);
-// Pairs (row, place) of the experts below `experts` gathered in tiles of leone_moe_tile_pairs() pairs of one expert:
-// tile_expert int32 [max_tiles] (-1: unused), tile_pairs int32 [max_tiles, tile pairs] (-1: empty);
-// max_tiles >= min(pairs, pairs / tile pairs + experts).
+// Pairs (row, place) of the experts below `experts` gathered in tiles of `tile` pairs of one expert (leone_moe_tile_pairs(),
+// 16, 64 or 128): tile_expert int32 [max_tiles] (-1: unused), tile_pairs int32 [max_tiles, tile] (-1: empty);
+// max_tiles >= min(pairs, pairs / tile + experts).
 int leone_moe_tile_pairs();
-int leone_moe_plan(const int* chosen, int pairs, int experts, int* tile_expert, int* tile_pairs, int max_tiles,
+int leone_moe_plan(const int* chosen, int pairs, int experts, int* tile_expert, int* tile_pairs, int max_tiles, int tile,
                    hipStream_t stream);
+// tile: leone_moe_tile_pairs() (any type and size), or 16, 64 or 128 (matrix cores: bfloat16, n and k multiples of 8).
 int leone_moe_product(const void* x, const void* w, void* y, const float* pair_weight, int dtype, int gated,
-                      const int* tile_expert, const int* tile_pairs, int max_tiles, int top, int n, int k, int act,
+                      const int* tile_expert, const int* tile_pairs, int max_tiles, int tile, int top, int n, int k, int act,
                       hipStream_t stream);
 int leone_moe_combine(const float* pair_out, const int* chosen, const float* weight, const void* x, int dtype,
                       const float* extra, float* out, int rows, int top, int experts, int hidden, hipStream_t stream);

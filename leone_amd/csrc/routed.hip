@@ -149,12 +149,12 @@ route_topk_kernel(const float* __restrict__ logits, AnyVec correction, int* __re
 // One workgroup.  counts and places live in shared memory (experts <= 1024).
 __global__ void __launch_bounds__(1024)
 moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int* __restrict__ tile_expert,
-                int* __restrict__ tile_pairs, int max_tiles) {
+                int* __restrict__ tile_pairs, int max_tiles, int tile) {
     __shared__ int count[1024];
     __shared__ int first_tile[1024];
     for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
     for (int t = threadIdx.x; t < max_tiles; t += blockDim.x) tile_expert[t] = -1;
-    for (long i = threadIdx.x; i < static_cast<long>(max_tiles) * kTilePairs; i += blockDim.x) tile_pairs[i] = -1;
+    for (long i = threadIdx.x; i < static_cast<long>(max_tiles) * tile; i += blockDim.x) tile_pairs[i] = -1;
     __syncthreads();
     for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
         const int e = chosen[p];
@@ -165,7 +165,7 @@ moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int* __r
         int at = 0;
         for (int e = 0; e < experts; ++e) {
             first_tile[e] = at;
-            const int tiles = (count[e] + kTilePairs - 1) / kTilePairs;
+            const int tiles = (count[e] + tile - 1) / tile;
             for (int t = 0; t < tiles && at + t < max_tiles; ++t) tile_expert[at + t] = e;
             at += tiles;
             count[e] = 0;
@@ -177,8 +177,8 @@ moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int* __r
         const int e = chosen[p];
         if (e >= 0 && e < experts) {
             const int at = atomicAdd(&count[e], 1);
-            const long place = static_cast<long>(first_tile[e]) * kTilePairs + at;
-            if (place < static_cast<long>(max_tiles) * kTilePairs) tile_pairs[place] = p;
+            const long place = static_cast<long>(first_tile[e]) * tile + at;
+            if (place < static_cast<long>(max_tiles) * tile) tile_pairs[place] = p;
         }
     }
 }
@@ -302,27 +302,286 @@ moe_product_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __res
     }
 }
 
-// One workgroup a row.
+
+// The same products on the matrix cores, bfloat16: a workgroup takes a tile of 16 * kPB pairs of one expert and 64
+// rows of its matrix, a wave 16 of those rows against all the tile's pairs (v_mfma_f32_16x16x32_bf16: the rows are
+// one operand, 16 pairs the other; lane (c, g) holds elements 8 g .. 8 g + 7 of a step of 32 of row c and of pair c,
+// and gets rows 4 g .. 4 g + 3 of pair c).  Inner sizes are multiples of 8; a step's lanes beyond the inner size
+// bring zeros.
+typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float moe_floatx4 __attribute__((ext_vector_type(4)));
+
+__device__ inline moe_bf16x8 moe_load8(const bf16_t* p) {
+    return __builtin_bit_cast(moe_bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+__device__ inline moe_bf16x8 moe_zero8() {
+    const uint4 z = {0u, 0u, 0u, 0u};
+    return __builtin_bit_cast(moe_bf16x8, z);
+}
+
+template <int kPB, int kRT, bool kGated>
+__global__ void __launch_bounds__(kMoeThreads)
+moe_product_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y,
+                        const float* __restrict__ pair_weight, const int* __restrict__ tile_expert,
+                        const int* __restrict__ tile_pairs, int top, int n, int k, int act) {
+    // kPB blocks of 16 pairs a tile; kRT blocks of 16 rows a wave (a workgroup takes 64 * kRT rows): the more of
+    // both, the fewer times the rows of the matrix and of x are fetched again by other workgroups.
+    constexpr int kTile = 16 * kPB;
+    const int tile = blockIdx.x;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int row0 = (blockIdx.y * kMoeWaves + wave) * 16 * kRT;
+    if (row0 >= n) return;
+    int pair[kPB];
+    const bf16_t* xrow[kPB];
+#pragma unroll
+    for (int b = 0; b < kPB; ++b) {
+        pair[b] = tile_pairs[static_cast<long>(tile) * kTile + 16 * b + c];
+        xrow[b] = x + static_cast<long>(pair[b] < 0 ? 0 : (kGated ? pair[b] / top : pair[b])) * k;
+    }
+    const long matrix = static_cast<long>(n) * k;
+    bool row_ok[kRT];
+    const bf16_t* wa[kRT];
+#pragma unroll
+    for (int t = 0; t < kRT; ++t) {
+        row_ok[t] = row0 + 16 * t + c < n;
+        wa[t] = w + static_cast<long>(e) * (kGated ? 2 : 1) * matrix + static_cast<long>(row_ok[t] ? row0 + 16 * t + c : 0) * k;
+    }
+    moe_floatx4 acc[kRT][kPB], acc2[kGated ? kRT : 1][kPB];
+#pragma unroll
+    for (int t = 0; t < kRT; ++t)
+#pragma unroll
+        for (int b = 0; b < kPB; ++b) {
+            acc[t][b] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+            if constexpr (kGated) acc2[t][b] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+    // A ring of kDepth steps of 32: a step's operands are asked for kDepth steps before the matrix instructions
+    // that use them run, so that a wave that has its SIMD to itself still keeps loads on their way.
+    constexpr int kDepth = kPB * kRT >= 16 ? 4 : kPB >= 4 ? 4 : 8;
+    moe_bf16x8 a[kDepth][kRT], a2[kDepth][kGated ? kRT : 1], xb[kDepth][kPB];
+#define LEONE_MOE_FETCH(D, K0)                                                                                  \
+    {                                                                                                           \
+        const int at = (K0) + 8 * g;                                                                            \
+        const bool in = at < k;                                                                                 \
+        _Pragma("unroll") for (int t = 0; t < kRT; ++t) {                                                       \
+            a[D][t] = (row_ok[t] && in) ? moe_load8(wa[t] + at) : moe_zero8();                                  \
+            if constexpr (kGated) a2[D][t] = (row_ok[t] && in) ? moe_load8(wa[t] + matrix + at) : moe_zero8();  \
+        }                                                                                                       \
+        _Pragma("unroll") for (int b = 0; b < kPB; ++b)                                                         \
+            xb[D][b] = (pair[b] >= 0 && in) ? moe_load8(xrow[b] + at) : moe_zero8();                            \
+    }
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) LEONE_MOE_FETCH(d, 32 * d)
+    for (int k0 = 0; k0 < k; k0 += 32 * kDepth) {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            if (k0 + 32 * d < k) {                                   // the same for the whole workgroup
+#pragma unroll
+                for (int t = 0; t < kRT; ++t) {
+#pragma unroll
+                    for (int b = 0; b < kPB; ++b) {
+                        acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[d][t], xb[d][b], acc[t][b], 0, 0, 0);
+                        if constexpr (kGated)
+                            acc2[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[d][t], xb[d][b], acc2[t][b], 0, 0, 0);
+                    }
+                }
+            }
+            LEONE_MOE_FETCH(d, k0 + 32 * (kDepth + d))
+        }
+    }
+#undef LEONE_MOE_FETCH
+#pragma unroll
+    for (int b = 0; b < kPB; ++b) {
+        if (pair[b] < 0) continue;
+        const float scale = kGated ? 1.f : pair_weight[pair[b]];
+#pragma unroll
+        for (int t = 0; t < kRT; ++t) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int r = row0 + 16 * t + 4 * g + j;
+                if (r >= n) continue;
+                if constexpr (kGated)
+                    static_cast<bf16_t*>(y)[static_cast<long>(pair[b]) * n + r] =
+                        from_float<bf16_t>(gate_act(acc[t][b][j], act) * acc2[t][b][j]);
+                else
+                    static_cast<float*>(y)[static_cast<long>(pair[b]) * n + r] = acc[t][b][j] * scale;
+            }
+        }
+    }
+}
+
+// Tiles of 128 pairs, bfloat16: a workgroup takes a tile and 128 rows of its expert's matrix (gated: 128 gate rows and
+// their up rows), in chunks of 64 of the inner size that go through shared memory: a row's chunk is one line of 128
+// bytes, fetched whole by eight neighbouring threads (rows of a matrix lie a power of two apart, so lines that are
+// only half used at a time push one another out of the caches before their other half is asked for).  While the
+// waves work on a chunk the next is on its way from memory into registers.  In shared memory a chunk lies as two
+// halves of 32 elements, rows one after the other within a half: the 16 rows of an operand are one kilobyte that the
+// 64 lanes read in one piece.  The four waves take 64 rows x 64 pairs each: 4 + 4 operands for 16 matrix instructions.
+constexpr int kBigPairs = 128;
+constexpr int kBigRows = 128;
+constexpr int kBigChunk = 64;
+
+template <bool kGated>
+__global__ void __launch_bounds__(kMoeThreads)
+moe_product_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y,
+                         const float* __restrict__ pair_weight, const int* __restrict__ tile_expert,
+                         const int* __restrict__ tile_pairs, int top, int n, int k, int act) {
+    constexpr int kWRows = kGated ? 2 * kBigRows : kBigRows;          // rows of the matrix in a chunk
+    constexpr int kXPieces = kBigPairs * 8 / kMoeThreads;             // 16-byte pieces of x a thread brings per chunk
+    constexpr int kWPieces = kWRows * 8 / kMoeThreads;
+    __shared__ uint4 sx[2 * kBigPairs * 4];                           // [half][row][4 pieces]
+    __shared__ uint4 sw[2 * kWRows * 4];
+    const int tile = blockIdx.x;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave, lane = tid % kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int wr = wave >> 1, wp = wave & 1;
+    const int row_base = blockIdx.y * kBigRows;
+    const long matrix = static_cast<long>(n) * k;
+    const int* my_pairs = tile_pairs + static_cast<long>(tile) * kBigPairs;
+
+    // what this thread brings: piece p = tid + 256 i is part p % 8 of row p / 8 (row tid / 8 + 32 i)
+    const int part = tid & 7;
+    const int half = part >> 2, quarter = part & 3;
+    const bf16_t* x_from[kXPieces];
+    const bf16_t* w_from[kWPieces];
+#pragma unroll
+    for (int i = 0; i < kXPieces; ++i) {
+        const int pair = my_pairs[tid / 8 + 32 * i];
+        x_from[i] = pair < 0 ? nullptr : x + static_cast<long>(kGated ? pair / top : pair) * k + 8 * part;
+    }
+#pragma unroll
+    for (int i = 0; i < kWPieces; ++i) {
+        const int local = tid / 8 + 32 * i;                           // gated: rows 0..127 gate, 128..255 up
+        const int row = row_base + (local % kBigRows);
+        w_from[i] = row >= n ? nullptr
+                             : w + static_cast<long>(e) * (kGated ? 2 : 1) * matrix + (local >= kBigRows ? matrix : 0) +
+                                   static_cast<long>(row) * k + 8 * part;
+    }
+    uint4 hx[kXPieces], hw[kWPieces];
+
+    moe_floatx4 acc[4][4], acc2[kGated ? 4 : 1][4];
+#pragma unroll
+    for (int ta = 0; ta < 4; ++ta)
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb) {
+            acc[ta][tb] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+            if constexpr (kGated) acc2[ta][tb] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+    const int chunks = (k + kBigChunk - 1) / kBigChunk;
+#define LEONE_MOE_BRING(K0)                                                                                              \
+    {                                                                                                                    \
+        const bool in = (K0) + 8 * part < k;                                                                             \
+        _Pragma("unroll") for (int i = 0; i < kXPieces; ++i) {                                                           \
+            hx[i] = uint4{0u, 0u, 0u, 0u};                                                                               \
+            if (x_from[i] && in) hx[i] = *reinterpret_cast<const uint4*>(x_from[i] + (K0));                              \
+        }                                                                                                                \
+        _Pragma("unroll") for (int i = 0; i < kWPieces; ++i) {                                                           \
+            hw[i] = uint4{0u, 0u, 0u, 0u};                                                                               \
+            if (w_from[i] && in) hw[i] = *reinterpret_cast<const uint4*>(w_from[i] + (K0));                              \
+        }                                                                                                                \
+    }
+    LEONE_MOE_BRING(0)
+    for (int ck = 0; ck < chunks; ++ck) {
+#pragma unroll
+        for (int i = 0; i < kXPieces; ++i) sx[(half * kBigPairs + tid / 8 + 32 * i) * 4 + quarter] = hx[i];
+#pragma unroll
+        for (int i = 0; i < kWPieces; ++i) sw[(half * kWRows + tid / 8 + 32 * i) * 4 + quarter] = hw[i];
+        __syncthreads();
+        if (ck + 1 < chunks) LEONE_MOE_BRING((ck + 1) * kBigChunk)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            moe_bf16x8 a[4], a2[kGated ? 4 : 1], b[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                a[t] = __builtin_bit_cast(moe_bf16x8, sw[(h * kWRows + 64 * wr + 16 * t + c) * 4 + g]);
+                if constexpr (kGated) a2[t] = __builtin_bit_cast(moe_bf16x8, sw[(h * kWRows + kBigRows + 64 * wr + 16 * t + c) * 4 + g]);
+                b[t] = __builtin_bit_cast(moe_bf16x8, sx[(h * kBigPairs + 64 * wp + 16 * t + c) * 4 + g]);
+            }
+#pragma unroll
+            for (int ta = 0; ta < 4; ++ta)
+#pragma unroll
+                for (int tb = 0; tb < 4; ++tb) {
+                    acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ta], b[tb], acc[ta][tb], 0, 0, 0);
+                    if constexpr (kGated) acc2[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[ta], b[tb], acc2[ta][tb], 0, 0, 0);
+                }
+        }
+        __syncthreads();                               // everyone has read the chunk before the next is put down
+    }
+#undef LEONE_MOE_BRING
+    // lane (c, g) holds rows 4 g .. 4 g + 3 of pair c of every (ta, tb)
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+        const int pair = my_pairs[64 * wp + 16 * tb + c];
+        if (pair < 0) continue;
+        const float scale = kGated ? 1.f : pair_weight[pair];
+#pragma unroll
+        for (int ta = 0; ta < 4; ++ta) {
+            const int r = row_base + 64 * wr + 16 * ta + 4 * g;
+            if (r >= n) continue;
+            float v0, v1, v2, v3;
+            if constexpr (kGated) {
+                v0 = gate_act(acc[ta][tb][0], act) * acc2[ta][tb][0];
+                v1 = gate_act(acc[ta][tb][1], act) * acc2[ta][tb][1];
+                v2 = gate_act(acc[ta][tb][2], act) * acc2[ta][tb][2];
+                v3 = gate_act(acc[ta][tb][3], act) * acc2[ta][tb][3];
+                bf16_t* to = static_cast<bf16_t*>(y) + static_cast<long>(pair) * n + r;
+                if (r + 3 < n && n % 4 == 0) {
+                    uint2 packed;
+                    packed.x = bf16_bits_from_float(v0) | (static_cast<uint32_t>(bf16_bits_from_float(v1)) << 16);
+                    packed.y = bf16_bits_from_float(v2) | (static_cast<uint32_t>(bf16_bits_from_float(v3)) << 16);
+                    *reinterpret_cast<uint2*>(to) = packed;
+                } else {
+                    to[0] = from_float<bf16_t>(v0);
+                    if (r + 1 < n) to[1] = from_float<bf16_t>(v1);
+                    if (r + 2 < n) to[2] = from_float<bf16_t>(v2);
+                    if (r + 3 < n) to[3] = from_float<bf16_t>(v3);
+                }
+            } else {
+                v0 = acc[ta][tb][0] * scale;
+                v1 = acc[ta][tb][1] * scale;
+                v2 = acc[ta][tb][2] * scale;
+                v3 = acc[ta][tb][3] * scale;
+                float* to = static_cast<float*>(y) + static_cast<long>(pair) * n + r;
+                if (r + 3 < n && n % 4 == 0) {
+                    *reinterpret_cast<float4*>(to) = float4{v0, v1, v2, v3};
+                } else {
+                    to[0] = v0;
+                    if (r + 1 < n) to[1] = v1;
+                    if (r + 2 < n) to[2] = v2;
+                    if (r + 3 < n) to[3] = v3;
+                }
+            }
+        }
+    }
+}
+
+// A workgroup takes 256 columns of a row; a thread one column.
 template <typename T>
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const float* __restrict__ pair_out, const int* __restrict__ chosen, const float* __restrict__ weight,
                    const T* __restrict__ x, const float* __restrict__ extra, float* __restrict__ out, int top, int experts,
                    int hidden) {
     const int row = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= hidden) return;
     const int* ch = chosen + static_cast<long>(row) * top;
     const float* wt = weight + static_cast<long>(row) * top;
-    for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
-        float sum = 0.f;
-        for (int j = 0; j < top; ++j) {
-            const int e = ch[j];
-            if (e >= experts)
-                sum += wt[j] * to_float(x[static_cast<long>(row) * hidden + c]);    // hands the row on as it came
-            else if (e >= 0)
-                sum += pair_out[(static_cast<long>(row) * top + j) * hidden + c];
-        }
-        if (extra != nullptr) sum += extra[static_cast<long>(row) * hidden + c];
-        out[static_cast<long>(row) * hidden + c] = sum;
+    const long at = static_cast<long>(row) * hidden + c;
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) {                       // in the order of the row's places, whatever the tiles were
+        const int e = ch[j];
+        if (e >= experts)
+            sum += wt[j] * to_float(x[at]);               // hands the row on as it came
+        else if (e >= 0)
+            sum += pair_out[(static_cast<long>(row) * top + j) * hidden + c];
     }
+    if (extra != nullptr) sum += extra[at];
+    out[at] = sum;
 }
 
 }  // namespace leone
@@ -348,22 +607,54 @@ extern "C" int leone_route_topk(const float* logits, const void* correction, int
 }
 
 extern "C" int leone_moe_plan(const int* chosen, int pairs, int experts, int* tile_expert, int* tile_pairs, int max_tiles,
-                              hipStream_t stream) {
+                              int tile, hipStream_t stream) {
+    LEONE_REQUIRE(tile == kTilePairs || tile == 16 || tile == 64 || tile == 128, "moe_plan: tiles of %d pairs", tile);
     LEONE_REQUIRE(chosen && tile_expert && tile_pairs, "moe_plan: null pointer");
     LEONE_REQUIRE(pairs > 0 && experts > 0 && experts <= 1024, "moe_plan: %d pairs, %d experts (at most 1024)", pairs, experts);
-    const long needed = static_cast<long>(pairs) / kTilePairs + experts;
+    const long needed = static_cast<long>(pairs) / tile + experts;
     LEONE_REQUIRE(max_tiles >= (needed < pairs ? needed : pairs), "moe_plan: %d tiles cannot hold %d pairs of %d experts", max_tiles,
                   pairs, experts);
-    moe_plan_kernel<<<1, 1024, 0, stream>>>(chosen, pairs, experts, tile_expert, tile_pairs, max_tiles);
+    moe_plan_kernel<<<1, 1024, 0, stream>>>(chosen, pairs, experts, tile_expert, tile_pairs, max_tiles, tile);
     LEONE_LAUNCH_CHECK("moe_plan");
     return 0;
 }
 
 // gated != 0: x [rows, k], w [experts, 2, n, k], y [pairs, n] of dtype = act(gate) * up (act: GateAct).
 // gated == 0: x [pairs, k], w [experts, n, k], y float32 [pairs, n] = pair_weight[pair] * product.
+// tile: pairs a tile holds, as leone_moe_plan was told: leone_moe_tile_pairs() for the kernel that takes any type and
+// size; 16 or 64 for the matrix-core kernel (bfloat16, n and k multiples of 8).
 extern "C" int leone_moe_product(const void* x, const void* w, void* y, const float* pair_weight, int dtype, int gated,
-                                 const int* tile_expert, const int* tile_pairs, int max_tiles, int top, int n, int k, int act,
-                                 hipStream_t stream) {
+                                 const int* tile_expert, const int* tile_pairs, int max_tiles, int tile, int top, int n, int k,
+                                 int act, hipStream_t stream) {
+    if (tile != kTilePairs) {
+        LEONE_REQUIRE(tile == 16 || tile == 64 || tile == 128, "moe_product: tiles of %d pairs", tile);
+        LEONE_REQUIRE(dtype == kBF16 && k % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
+                      "moe_product: the matrix-core kernel takes bfloat16 with an inner size that is a multiple of 8, not %d", k);
+        LEONE_REQUIRE(x && w && y && tile_expert && tile_pairs && (gated || pair_weight), "moe_product: null pointer");
+        LEONE_REQUIRE(max_tiles > 0 && top > 0 && n > 0 && k > 0, "moe_product: %d tiles, sizes %d x %d", max_tiles, n, k);
+        LEONE_REQUIRE(act == kGateSilu || act == kGateGeluTanh, "moe_product: unknown activation %d", act);
+        const dim3 cores(max_tiles, ceil_div(n, tile == 128 ? 128 : 64));
+        LEONE_REQUIRE(cores.y <= 65535, "moe_product: %d rows of a matrix are too many", n);
+#define LEONE_MOE_CORES(PB, RT, G)                                                                                      \
+    moe_product_mfma_kernel<PB, RT, G><<<cores, kMoeThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), \
+                                                                          y, pair_weight, tile_expert, tile_pairs, top, n, k, act)
+        if (tile == 16) {
+            if (gated) LEONE_MOE_CORES(1, 1, true);
+            else LEONE_MOE_CORES(1, 1, false);
+        } else if (tile == 64) {
+            if (gated) LEONE_MOE_CORES(4, 1, true);
+            else LEONE_MOE_CORES(4, 1, false);
+        } else if (gated) {
+            moe_product_tiled_kernel<true><<<cores, kMoeThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y,
+                                                                              pair_weight, tile_expert, tile_pairs, top, n, k, act);
+        } else {
+            moe_product_tiled_kernel<false><<<cores, kMoeThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y,
+                                                                               pair_weight, tile_expert, tile_pairs, top, n, k, act);
+        }
+#undef LEONE_MOE_CORES
+        LEONE_LAUNCH_CHECK("moe_product");
+        return 0;
+    }
     LEONE_REQUIRE(dtype == kF32 || dtype == kBF16, "moe_product: unknown element type %d", dtype);
     LEONE_REQUIRE(x && w && y && tile_expert && tile_pairs && (gated || pair_weight), "moe_product: null pointer");
     LEONE_REQUIRE(max_tiles > 0 && top > 0 && n > 0 && k > 0, "moe_product: %d tiles, sizes %d x %d", max_tiles, n, k);
@@ -392,11 +683,13 @@ extern "C" int leone_moe_combine(const float* pair_out, const int* chosen, const
     LEONE_REQUIRE(dtype == kF32 || dtype == kBF16, "moe_combine: unknown element type %d", dtype);
     LEONE_REQUIRE(pair_out && chosen && weight && x && out, "moe_combine: null pointer");
     LEONE_REQUIRE(rows > 0 && top > 0 && experts >= 0 && hidden > 0, "moe_combine: rows %d, top %d, hidden %d", rows, top, hidden);
+    const dim3 grid(rows, ceil_div(hidden, 256));
+    LEONE_REQUIRE(grid.y <= 65535, "moe_combine: rows of %d are too wide", hidden);
     if (dtype == kF32)
-        moe_combine_kernel<float><<<rows, 256, 0, stream>>>(pair_out, chosen, weight, static_cast<const float*>(x), extra, out, top,
+        moe_combine_kernel<float><<<grid, 256, 0, stream>>>(pair_out, chosen, weight, static_cast<const float*>(x), extra, out, top,
                                                             experts, hidden);
     else
-        moe_combine_kernel<bf16_t><<<rows, 256, 0, stream>>>(pair_out, chosen, weight, static_cast<const bf16_t*>(x), extra, out, top,
+        moe_combine_kernel<bf16_t><<<grid, 256, 0, stream>>>(pair_out, chosen, weight, static_cast<const bf16_t*>(x), extra, out, top,
                                                              experts, hidden);
     LEONE_LAUNCH_CHECK("moe_combine");
     return 0;

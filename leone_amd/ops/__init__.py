@@ -1479,6 +1479,9 @@ def route_topk(logits: torch.Tensor, correction: Optional[torch.Tensor], top: in
     return chosen, weight
 
 
+MOE_WIDE_TILE_PAIRS = 32      # from this many (row, place) pairs an expert on average, the experts' products take tiles of 64 pairs
+
+
 def routed_experts(x: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, w_gate_up: torch.Tensor,
                    w_down: torch.Tensor, activation: str = "silu", extra: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Every row through the experts chosen for it: float32 ``[rows, hidden]`` = sum over a row's places of
@@ -1493,21 +1496,26 @@ def routed_experts(x: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, 
         raise KernelError(f"routed_experts: matrices {tuple(w_gate_up.shape)} and {tuple(w_down.shape)} of {w_gate_up.dtype} "
                           f"do not fit rows {tuple(x.shape)} of {x.dtype}")
     pairs = rows * top
-    tile = library().leone_moe_tile_pairs()
+    # bfloat16 with inner sizes in runs of 8 goes to the matrix cores: tiles of 128 or 64 pairs where an expert gets
+    # many (its matrices are read once a tile), of 16 where it gets few; anything else in tiles of the plain kernel's size
+    if x.dtype == torch.bfloat16 and hidden % 8 == 0 and ff % 8 == 0:
+        tile = 128 if pairs >= 4 * MOE_WIDE_TILE_PAIRS * experts else 64 if pairs >= MOE_WIDE_TILE_PAIRS * experts else 16
+    else:
+        tile = library().leone_moe_tile_pairs()
     max_tiles = min(pairs, pairs // tile + experts)
     device = x.device
     tile_expert = torch.empty((max_tiles,), dtype=torch.int32, device=device)
     tile_pairs = torch.empty((max_tiles, tile), dtype=torch.int32, device=device)
     call("leone_moe_plan", _dev(chosen, "chosen", torch.int32, (rows, top)), pairs, experts, _dev(tile_expert, "tiles"),
-         _dev(tile_pairs, "tile pairs"), max_tiles, _stream())
+         _dev(tile_pairs, "tile pairs"), max_tiles, tile, _stream())
     hidden_act = torch.empty((pairs, ff), dtype=x.dtype, device=device)
     call("leone_moe_product", _dev(x, "routed rows"), _dev(w_gate_up, "expert gate/up"), _dev(hidden_act, "expert hidden"), 0,
-         _code(x, "routed rows"), 1, _dev(tile_expert, "tiles"), _dev(tile_pairs, "tile pairs"), max_tiles, top, ff, hidden,
+         _code(x, "routed rows"), 1, _dev(tile_expert, "tiles"), _dev(tile_pairs, "tile pairs"), max_tiles, tile, top, ff, hidden,
          _gate_code(activation), _stream())
     pair_out = torch.empty((pairs, hidden), dtype=torch.float32, device=device)
     call("leone_moe_product", _dev(hidden_act, "expert hidden"), _dev(w_down, "expert down"), _dev(pair_out, "pair results"),
          _dev(weight, "weights", torch.float32, (rows, top)), _code(x, "routed rows"), 0, _dev(tile_expert, "tiles"),
-         _dev(tile_pairs, "tile pairs"), max_tiles, top, hidden, ff, 0, _stream())
+         _dev(tile_pairs, "tile pairs"), max_tiles, tile, top, hidden, ff, 0, _stream())
     out = torch.empty((rows, hidden), dtype=torch.float32, device=device)
     call("leone_moe_combine", _dev(pair_out, "pair results"), _dev(chosen, "chosen"), _dev(weight, "weights"),
          _dev(x, "routed rows"), _code(x, "routed rows"), _dev(extra, "extra", torch.float32, (rows, hidden)),
