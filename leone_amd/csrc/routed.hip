@@ -40,18 +40,17 @@ __device__ inline void wave_best(float& v, int& at) {
     }
 }
 
-// One wave a row.
-__global__ void __launch_bounds__(kWave)
-route_topk_kernel(const float* __restrict__ logits, AnyVec correction, int* __restrict__ chosen, float* __restrict__ weight,
-                  int total, int top, int group_count, int group_keep) {
-    const int row = blockIdx.x;
-    const int lane = threadIdx.x;
+// One wave a row; a lane holds kSlots router outputs (kSlots * 64 >= total).
+template <int kSlots>
+__device__ inline void route_row(int row, int lane, const float* __restrict__ logits, const AnyVec& correction,
+                                 int* __restrict__ chosen, float* __restrict__ weight, int total, int top, int group_count,
+                                 int group_keep) {
     const float* z = logits + static_cast<long>(row) * total;
-    float s[kRouteSlots], choice[kRouteSlots];
-    bool taken[kRouteSlots];
+    float s[kSlots], choice[kSlots];
+    bool taken[kSlots];
     float top_z = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < kRouteSlots; ++i) {
+    for (int i = 0; i < kSlots; ++i) {
         const int e = lane + i * kWave;
         s[i] = e < total ? z[e] : -INFINITY;
         top_z = fmaxf(top_z, s[i]);
@@ -59,14 +58,14 @@ route_topk_kernel(const float* __restrict__ logits, AnyVec correction, int* __re
     top_z = wave_max(top_z);
     float sum = 0.f;
 #pragma unroll
-    for (int i = 0; i < kRouteSlots; ++i) {
+    for (int i = 0; i < kSlots; ++i) {
         const int e = lane + i * kWave;
         s[i] = e < total ? expf(s[i] - top_z) : 0.f;
         sum += s[i];
     }
     sum = wave_sum(sum);
 #pragma unroll
-    for (int i = 0; i < kRouteSlots; ++i) {
+    for (int i = 0; i < kSlots; ++i) {
         const int e = lane + i * kWave;
         s[i] = s[i] / sum;
         choice[i] = e < total ? s[i] + (correction.ptr ? load_any(correction, e) : 0.f) : -INFINITY;
@@ -75,13 +74,16 @@ route_topk_kernel(const float* __restrict__ logits, AnyVec correction, int* __re
     if (group_count > 1) {
         // a group's score; lane g keeps group g's (group_count <= 64)
         const int size = total / group_count;
+        int group_of[kSlots];
+#pragma unroll
+        for (int i = 0; i < kSlots; ++i) group_of[i] = (lane + i * kWave) / size;
         float mine = -INFINITY;
         for (int g = 0; g < group_count; ++g) {
             float best = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < kRouteSlots; ++i) {
+            for (int i = 0; i < kSlots; ++i) {
                 const int e = lane + i * kWave;
-                if (e < total && e / size == g) best = fmaxf(best, choice[i]);
+                if (e < total && group_of[i] == g) best = fmaxf(best, choice[i]);
             }
             best = wave_max(best);
             if (lane == g) mine = best;
@@ -97,9 +99,9 @@ route_topk_kernel(const float* __restrict__ logits, AnyVec correction, int* __re
             if (lane == at) mine_taken = true;
         }
 #pragma unroll
-        for (int i = 0; i < kRouteSlots; ++i) {
+        for (int i = 0; i < kSlots; ++i) {
             const int e = lane + i * kWave;
-            if (e < total && !((open >> (e / size)) & 1ull)) choice[i] = -INFINITY;
+            if (e < total && !((open >> group_of[i]) & 1ull)) choice[i] = -INFINITY;
         }
     }
     float picked_sum = 0.f;
@@ -109,7 +111,7 @@ route_topk_kernel(const float* __restrict__ logits, AnyVec correction, int* __re
         float v = -INFINITY;
         int at = 0x7fffffff;
 #pragma unroll
-        for (int i = 0; i < kRouteSlots; ++i) {
+        for (int i = 0; i < kSlots; ++i) {
             const int e = lane + i * kWave;
             if (!taken[i] && (at == 0x7fffffff || choice[i] > v)) {
                 v = choice[i];
@@ -119,7 +121,7 @@ route_topk_kernel(const float* __restrict__ logits, AnyVec correction, int* __re
         wave_best(v, at);
         float got = 0.f;
 #pragma unroll
-        for (int i = 0; i < kRouteSlots; ++i) {
+        for (int i = 0; i < kSlots; ++i) {
             const int e = lane + i * kWave;
             if (e == at) {
                 taken[i] = true;
@@ -146,12 +148,17 @@ route_topk_kernel(const float* __restrict__ logits, AnyVec correction, int* __re
         for (int n = kWave; n < top; ++n) weight[static_cast<long>(row) * top + n] /= denom;
 }
 
+__global__ void __launch_bounds__(kWave)
+route_topk_kernel(const float* __restrict__ logits, AnyVec correction, int* __restrict__ chosen, float* __restrict__ weight,
+                  int total, int top, int group_count, int group_keep) {
+    if (total <= kWave) route_row<1>(blockIdx.x, threadIdx.x, logits, correction, chosen, weight, total, top, group_count, group_keep);
+    else if (total <= 2 * kWave) route_row<2>(blockIdx.x, threadIdx.x, logits, correction, chosen, weight, total, top, group_count, group_keep);
+    else route_row<kRouteSlots>(blockIdx.x, threadIdx.x, logits, correction, chosen, weight, total, top, group_count, group_keep);
+}
+
 // One workgroup.  counts and places live in shared memory (experts <= 1024).
-__global__ void __launch_bounds__(1024)
-moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int* __restrict__ tile_expert,
-                int* __restrict__ tile_pairs, int max_tiles, int tile) {
-    __shared__ int count[1024];
-    __shared__ int first_tile[1024];
+__device__ inline void plan_tiles(const int* __restrict__ chosen, int pairs, int experts, int* __restrict__ tile_expert,
+                                  int* __restrict__ tile_pairs, int max_tiles, int tile, int* count, int* first_tile) {
     for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
     for (int t = threadIdx.x; t < max_tiles; t += blockDim.x) tile_expert[t] = -1;
     for (long i = threadIdx.x; i < static_cast<long>(max_tiles) * tile; i += blockDim.x) tile_pairs[i] = -1;
@@ -181,6 +188,31 @@ moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int* __r
             if (place < static_cast<long>(max_tiles) * tile) tile_pairs[place] = p;
         }
     }
+}
+
+__global__ void __launch_bounds__(1024)
+moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int* __restrict__ tile_expert,
+                int* __restrict__ tile_pairs, int max_tiles, int tile) {
+    __shared__ int count[1024];
+    __shared__ int first_tile[1024];
+    plan_tiles(chosen, pairs, experts, tile_expert, tile_pairs, max_tiles, tile, count, first_tile);
+}
+
+// The router's choice and the tiles in one launch, for steps of few rows (a wave a row, 16 waves in turn).
+__global__ void __launch_bounds__(1024)
+route_plan_kernel(const float* __restrict__ logits, AnyVec correction, int* __restrict__ chosen, float* __restrict__ weight,
+                  int rows, int total, int top, int group_count, int group_keep, int experts, int* __restrict__ tile_expert,
+                  int* __restrict__ tile_pairs, int max_tiles, int tile) {
+    __shared__ int count[1024];
+    __shared__ int first_tile[1024];
+    for (int row = threadIdx.x / kWave; row < rows; row += 1024 / kWave) {
+        const int lane = threadIdx.x % kWave;
+        if (total <= kWave) route_row<1>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep);
+        else if (total <= 2 * kWave) route_row<2>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep);
+        else route_row<kRouteSlots>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep);
+    }
+    __syncthreads();                                   // the choices are written; the same workgroup reads them
+    plan_tiles(chosen, rows * top, experts, tile_expert, tile_pairs, max_tiles, tile, count, first_tile);
 }
 
 template <typename T>
@@ -424,7 +456,7 @@ constexpr int kBigRows = 128;
 constexpr int kBigChunk = 64;
 
 template <bool kGated>
-__global__ void __launch_bounds__(kMoeThreads)
+__global__ void __launch_bounds__(kMoeThreads, 2)
 moe_product_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y,
                          const float* __restrict__ pair_weight, const int* __restrict__ tile_expert,
                          const int* __restrict__ tile_pairs, int top, int n, int k, int act) {
@@ -603,6 +635,29 @@ extern "C" int leone_route_topk(const float* logits, const void* correction, int
     route_topk_kernel<<<rows, kWave, 0, stream>>>(logits, AnyVec{correction, correction_dtype}, chosen, weight, total, top,
                                                   group_count, group_keep);
     LEONE_LAUNCH_CHECK("route_topk");
+    return 0;
+}
+
+// leone_route_topk and leone_moe_plan in one launch (one workgroup: for steps of few rows).
+extern "C" int leone_route_plan(const float* logits, const void* correction, int correction_dtype, int* chosen, float* weight,
+                                int rows, int total, int top, int group_count, int group_keep, int experts, int* tile_expert,
+                                int* tile_pairs, int max_tiles, int tile, hipStream_t stream) {
+    LEONE_REQUIRE(logits && chosen && weight && tile_expert && tile_pairs, "route_plan: null pointer");
+    LEONE_REQUIRE(rows > 0 && rows <= 256 && total > 0 && total <= kRouteSlots * kWave, "route_plan: rows %d (at most 256), %d router outputs",
+                  rows, total);
+    LEONE_REQUIRE(top > 0 && top <= total, "route_plan: %d of %d outputs", top, total);
+    LEONE_REQUIRE(!correction || correction_dtype == kF32 || correction_dtype == kBF16, "route_plan: unknown type of the correction");
+    LEONE_REQUIRE(group_count >= 1 && group_count <= kWave && total % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
+                  "route_plan: %d groups (at most %d, dividing %d outputs), %d kept", group_count, kWave, total, group_keep);
+    LEONE_REQUIRE(experts > 0 && experts <= 1024, "route_plan: %d experts (at most 1024)", experts);
+    LEONE_REQUIRE(tile == kTilePairs || tile == 16 || tile == 64 || tile == 128, "route_plan: tiles of %d pairs", tile);
+    const long pairs = static_cast<long>(rows) * top;
+    const long needed = pairs / tile + experts;
+    LEONE_REQUIRE(max_tiles >= (needed < pairs ? needed : pairs), "route_plan: %d tiles cannot hold %ld pairs of %d experts", max_tiles,
+                  pairs, experts);
+    route_plan_kernel<<<1, 1024, 0, stream>>>(logits, AnyVec{correction, correction_dtype}, chosen, weight, rows, total, top,
+                                              group_count, group_keep, experts, tile_expert, tile_pairs, max_tiles, tile);
+    LEONE_LAUNCH_CHECK("route_plan");
     return 0;
 }
 

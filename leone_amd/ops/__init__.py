@@ -1480,21 +1480,11 @@ def route_topk(logits: torch.Tensor, correction: Optional[torch.Tensor], top: in
 
 
 MOE_WIDE_TILE_PAIRS = 32      # from this many (row, place) pairs an expert on average, the experts' products take tiles of 64 pairs
+ROUTE_PLAN_ROWS = 64          # up to here the router's choice and the tiles are made in one launch
 
 
-def routed_experts(x: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, w_gate_up: torch.Tensor,
-                   w_down: torch.Tensor, activation: str = "silu", extra: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Every row through the experts chosen for it: float32 ``[rows, hidden]`` = sum over a row's places of
-    weight * W_down[e] (act(W_gate[e] x) * (W_up[e] x)), in the places' order; a chosen index from the number of
-    experts on stands for an expert that hands the row on as it is; ``extra`` (float32 ``[rows, hidden]``) is added.
-    ``w_gate_up`` is ``[experts, 2, ff, hidden]`` (gate rows, then up rows), ``w_down`` ``[experts, hidden, ff]``, both
-    of ``x``'s type.  Nothing here depends on the choice except through device arrays."""
-    rows, hidden = x.shape
-    top = chosen.shape[1]
-    experts, two, ff, k = w_gate_up.shape
-    if two != 2 or k != hidden or tuple(w_down.shape) != (experts, hidden, ff) or w_gate_up.dtype != x.dtype or w_down.dtype != x.dtype:
-        raise KernelError(f"routed_experts: matrices {tuple(w_gate_up.shape)} and {tuple(w_down.shape)} of {w_gate_up.dtype} "
-                          f"do not fit rows {tuple(x.shape)} of {x.dtype}")
+def _expert_tiles(x: torch.Tensor, rows: int, top: int, experts: int, hidden: int, ff: int):
+    """(pairs a tile, tiles at most, tile_expert, tile_pairs) for a step of ``rows`` rows."""
     pairs = rows * top
     # bfloat16 with inner sizes in runs of 8 goes to the matrix cores: tiles of 128 or 64 pairs where an expert gets
     # many (its matrices are read once a tile), of 16 where it gets few; anything else in tiles of the plain kernel's size
@@ -1503,11 +1493,25 @@ def routed_experts(x: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, 
     else:
         tile = library().leone_moe_tile_pairs()
     max_tiles = min(pairs, pairs // tile + experts)
+    return (tile, max_tiles, torch.empty((max_tiles,), dtype=torch.int32, device=x.device),
+            torch.empty((max_tiles, tile), dtype=torch.int32, device=x.device))
+
+
+def _check_experts(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor):
+    rows, hidden = x.shape
+    experts, two, ff, k = w_gate_up.shape
+    if two != 2 or k != hidden or tuple(w_down.shape) != (experts, hidden, ff) or w_gate_up.dtype != x.dtype or w_down.dtype != x.dtype:
+        raise KernelError(f"routed experts: matrices {tuple(w_gate_up.shape)} and {tuple(w_down.shape)} of {w_gate_up.dtype} "
+                          f"do not fit rows {tuple(x.shape)} of {x.dtype}")
+    return rows, hidden, experts, ff
+
+
+def _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, extra) -> torch.Tensor:
+    rows, hidden, experts, ff = _check_experts(x, w_gate_up, w_down)
+    top = chosen.shape[1]
+    pairs = rows * top
+    tile, max_tiles, tile_expert, tile_pairs = tiles
     device = x.device
-    tile_expert = torch.empty((max_tiles,), dtype=torch.int32, device=device)
-    tile_pairs = torch.empty((max_tiles, tile), dtype=torch.int32, device=device)
-    call("leone_moe_plan", _dev(chosen, "chosen", torch.int32, (rows, top)), pairs, experts, _dev(tile_expert, "tiles"),
-         _dev(tile_pairs, "tile pairs"), max_tiles, tile, _stream())
     hidden_act = torch.empty((pairs, ff), dtype=x.dtype, device=device)
     call("leone_moe_product", _dev(x, "routed rows"), _dev(w_gate_up, "expert gate/up"), _dev(hidden_act, "expert hidden"), 0,
          _code(x, "routed rows"), 1, _dev(tile_expert, "tiles"), _dev(tile_pairs, "tile pairs"), max_tiles, tile, top, ff, hidden,
@@ -1521,3 +1525,40 @@ def routed_experts(x: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, 
          _dev(x, "routed rows"), _code(x, "routed rows"), _dev(extra, "extra", torch.float32, (rows, hidden)),
          _dev(out, "routed out"), rows, top, experts, hidden, _stream())
     return out
+
+
+def routed_experts(x: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, w_gate_up: torch.Tensor,
+                   w_down: torch.Tensor, activation: str = "silu", extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Every row through the experts chosen for it: float32 ``[rows, hidden]`` = sum over a row's places of
+    weight * W_down[e] (act(W_gate[e] x) * (W_up[e] x)), in the places' order; a chosen index from the number of
+    experts on stands for an expert that hands the row on as it is; ``extra`` (float32 ``[rows, hidden]``) is added.
+    ``w_gate_up`` is ``[experts, 2, ff, hidden]`` (gate rows, then up rows), ``w_down`` ``[experts, hidden, ff]``, both
+    of ``x``'s type.  Nothing here depends on the choice except through device arrays."""
+    rows, hidden, experts, ff = _check_experts(x, w_gate_up, w_down)
+    top = chosen.shape[1]
+    tiles = _expert_tiles(x, rows, top, experts, hidden, ff)
+    call("leone_moe_plan", _dev(chosen, "chosen", torch.int32, (rows, top)), rows * top, experts, _dev(tiles[2], "tiles"),
+         _dev(tiles[3], "tile pairs"), tiles[1], tiles[0], _stream())
+    return _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, extra)
+
+
+def routed_feed_forward(x: torch.Tensor, logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, group_count: int,
+                        group_keep: int, w_gate_up: torch.Tensor, w_down: torch.Tensor, activation: str = "silu",
+                        extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``route_topk`` on the router's float32 ``logits`` and ``routed_experts`` with its choice; for steps of few rows
+    the choice and the tiles are made in one launch."""
+    rows, hidden, experts, ff = _check_experts(x, w_gate_up, w_down)
+    total = logits.shape[1]
+    if rows > ROUTE_PLAN_ROWS:
+        chosen, weight = route_topk(logits, correction, top, group_count, group_keep)
+        return routed_experts(x, chosen, weight, w_gate_up, w_down, activation, extra)
+    if total > library().leone_route_max_outputs():
+        raise KernelError(f"route_topk: {total} router outputs, the kernel takes {library().leone_route_max_outputs()}")
+    tiles = _expert_tiles(x, rows, top, experts, hidden, ff)
+    chosen = torch.empty((rows, top), dtype=torch.int32, device=x.device)
+    weight = torch.empty((rows, top), dtype=torch.float32, device=x.device)
+    call("leone_route_plan", _dev(logits, "router logits", torch.float32, (rows, total)),
+         _dev(correction, "router correction", None, (total,)), _code(correction, "router correction") if correction is not None else F32,
+         _dev(chosen, "chosen"), _dev(weight, "weights"), rows, total, int(top), int(group_count), int(group_keep), experts,
+         _dev(tiles[2], "tiles"), _dev(tiles[3], "tile pairs"), tiles[1], tiles[0], _stream())
+    return _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, extra)

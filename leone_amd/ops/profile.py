@@ -55,6 +55,7 @@ OPERATIONS = {
     "leone_attention_prefill_kept": "attention",
     "leone_route_topk": "router",
     "leone_moe_plan": "router",
+    "leone_route_plan": "router",
     "leone_moe_product": "experts",
     "leone_moe_combine": "experts",
 }

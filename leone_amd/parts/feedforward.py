@@ -159,7 +159,6 @@ class RoutedGluMlp(Part):
     def forward(self, y: torch.Tensor, step: StepContext) -> torch.Tensor:
         y = ops.materialize(y)
         logits = ops.linear(y, self.w_router, out_dtype=torch.float32)
-        chosen, weight = ops.route_topk(logits, self.correction, self.top, self.group_count, self.group_keep)
         extra = None
         if self.shared is not None:
             extra = self.shared.forward(y, step)
@@ -167,4 +166,5 @@ class RoutedGluMlp(Part):
                 extra = extra.sum(dim=0)
             if extra.dtype != torch.float32:
                 extra = extra.float()
-        return ops.routed_experts(y, chosen, weight, self.w_gate_up, self.w_down, self.activation, extra=extra)
+        return ops.routed_feed_forward(y, logits, self.correction, self.top, self.group_count, self.group_keep,
+                                       self.w_gate_up, self.w_down, self.activation, extra=extra)

@@ -273,6 +273,7 @@ ROUTERS = [{"experts": 6, "identity": 2, "top": 3, "groups": {"count": 4, "keep"
            {"experts": 5, "identity": 0, "top": 1},
            {"experts": 9, "identity": 1, "top": 4, "groups": {"count": 5, "keep": 3}},
            {"experts": 60, "identity": 12, "top": 6, "groups": {"count": 8, "keep": 3}},
+           {"experts": 140, "identity": 10, "top": 8, "groups": {"count": 10, "keep": 4}},
            {"experts": 4, "identity": 0, "top": 4, "groups": {"count": 1, "keep": 1}}]
 
 
@@ -321,6 +322,36 @@ def test_routed_experts(rows, sizes, dtype):
         for e, a in zip(chosen[t].tolist(), weight[t].double()):
             want[t] += a * (h[t].double() if e >= experts else plain.glu(h[t:t + 1].double(), wide, f"e{e}.", plain.silu)[0])
     close(out, want, 3e-6 if dtype == torch.float32 else 2e-2, f"{sizes} {rows} rows")
+
+
+@pytest.mark.parametrize("rows", [1, 9, 64, 65, 300])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mixture_part_against_plain(rows, dtype):
+    """The whole feed-forward part: router product, choice, tiles (in one launch up to 64 rows), experts, identity
+    experts and the shared expert, against the plain mixture; in bfloat16 rows whose choice is a close call are left
+    out of the comparison (the plain router sees the unrounded product)."""
+    from leone_amd.parts import FEED_FORWARDS, PartSpec
+    width = 64
+    mlp = zu.moe(6, 3, 24, identity=2, groups=(4, 2), shared=40)
+    raw = zu.config(width, 50, [zu.layer(zu.attention(2, 1, 8, 8), mlp)])
+    weights = {k[len("l0.mlp."):]: v for k, v in zu.make_weights(raw, 12, dtype).items() if k.startswith("l0.mlp.")}
+    shared = PartSpec("swiglu", {"hidden": width, "intermediate": 40, "float_output": True, "gate": "shared.gate",
+                                 "up": "shared.up", "down": "shared.down"})
+    part = FEED_FORWARDS.build(PartSpec("routed_glu", {"hidden": width, "experts": 6, "identity": 2, "top": 3, "group_count": 4,
+                                                       "group_keep": 2, "intermediate": 24, "router": "router",
+                                                       "correction": "correction", "expert": "e{e}", "shared": shared}))
+    part.bind({k: v.to(DEV) for k, v in weights.items()})
+    h = torch.randn(rows, width, generator=torch.Generator().manual_seed(rows)).to(dtype)
+    out = part.forward(h.to(DEV), None)
+    wide = {k: v.double() for k, v in weights.items()}
+    want = plain.mixture(h.double(), mlp, wide, "")
+    keep = torch.ones(rows, dtype=torch.bool)
+    if dtype == torch.bfloat16:
+        s = torch.softmax(h.double() @ wide["router"].T, dim=-1) + wide["correction"]
+        ranked = s.sort(dim=-1, descending=True).values
+        keep = (ranked[:, :-1] - ranked[:, 1:]).min(dim=-1).values > 2e-3      # no two choice scores close to each other
+        assert keep.sum() >= rows // 2
+    close(out.cpu()[keep], want[keep], 3e-6 if dtype == torch.float32 else 2e-2, f"mixture of {rows} rows")
 
 
 def planted(n, heads, dim, vdim, seed):
