@@ -204,6 +204,17 @@ class ZukinexConfig:
         return {"architecture": self.architecture, "vocab": self.vocab, "width": self.width,
                 "max_positions": self.max_positions, "norm": {"eps": self.eps}, "layers": layers}
 
+    # what the generic entry points ask a configuration for
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
+    @property
+    def max_position_embeddings(self) -> int:
+        return self.max_positions
+
+    eos_token_id = None
+
     def kv_retention(self, layer: int) -> Tuple[Optional[int], int]:
         """(window, keep_first) that the cache of ``layer`` must keep: the widest of its own mask and of the masks
         of the layers that read its keys and values (None: everything)."""

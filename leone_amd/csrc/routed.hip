@@ -72,12 +72,18 @@ __device__ inline void route_row(int row, int lane, const float* __restrict__ lo
         taken[i] = e >= total;
     }
     if (group_count > 1) {
-        // a group's score; lane g keeps group g's (group_count <= 64)
+        // a group's score: lane g % 64 keeps group g's in its place g / 64 (there are no more groups than outputs)
         const int size = total / group_count;
         int group_of[kSlots];
 #pragma unroll
         for (int i = 0; i < kSlots; ++i) group_of[i] = (lane + i * kWave) / size;
-        float mine = -INFINITY;
+        float mine[kSlots];
+        bool mine_taken[kSlots];
+#pragma unroll
+        for (int i = 0; i < kSlots; ++i) {
+            mine[i] = -INFINITY;
+            mine_taken[i] = lane + i * kWave >= group_count;
+        }
         for (int g = 0; g < group_count; ++g) {
             float best = -INFINITY;
 #pragma unroll
@@ -86,22 +92,35 @@ __device__ inline void route_row(int row, int lane, const float* __restrict__ lo
                 if (e < total && group_of[i] == g) best = fmaxf(best, choice[i]);
             }
             best = wave_max(best);
-            if (lane == g) mine = best;
+#pragma unroll
+            for (int i = 0; i < kSlots; ++i)
+                if (lane + i * kWave == g) mine[i] = best;
         }
-        unsigned long long open = 0ull;
-        bool mine_taken = lane >= group_count;
+        unsigned open = 0u;                                   // bit i: group lane + 64 i stays open
         for (int n = 0; n < group_keep; ++n) {
-            float v = mine_taken ? -INFINITY : mine;
-            int at = mine_taken ? 0x7fffffff : lane;
+            float v = -INFINITY;
+            int at = 0x7fffffff;
+#pragma unroll
+            for (int i = 0; i < kSlots; ++i)
+                if (!mine_taken[i] && (at == 0x7fffffff || mine[i] > v)) {
+                    v = mine[i];
+                    at = lane + i * kWave;
+                }
             wave_best(v, at);
             if (at == 0x7fffffff) break;
-            open |= 1ull << at;
-            if (lane == at) mine_taken = true;
+#pragma unroll
+            for (int i = 0; i < kSlots; ++i)
+                if (lane + i * kWave == at) {
+                    mine_taken[i] = true;
+                    open |= 1u << i;
+                }
         }
 #pragma unroll
         for (int i = 0; i < kSlots; ++i) {
             const int e = lane + i * kWave;
-            if (e < total && !((open >> group_of[i]) & 1ull)) choice[i] = -INFINITY;
+            const int g = e < total ? group_of[i] : 0;
+            const unsigned theirs = __shfl(open, g % kWave, kWave);
+            if (e < total && !((theirs >> (g / kWave)) & 1u)) choice[i] = -INFINITY;
         }
     }
     float picked_sum = 0.f;
@@ -630,8 +649,8 @@ extern "C" int leone_route_topk(const float* logits, const void* correction, int
                   rows, total, kRouteSlots * kWave);
     LEONE_REQUIRE(top > 0 && top <= total, "route_topk: %d of %d outputs", top, total);
     LEONE_REQUIRE(!correction || correction_dtype == kF32 || correction_dtype == kBF16, "route_topk: unknown type of the correction");
-    LEONE_REQUIRE(group_count >= 1 && group_count <= kWave && total % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
-                  "route_topk: %d groups (at most %d, dividing %d outputs), %d kept", group_count, kWave, total, group_keep);
+    LEONE_REQUIRE(group_count >= 1 && total % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
+                  "route_topk: %d groups (dividing %d outputs), %d kept", group_count, total, group_keep);
     route_topk_kernel<<<rows, kWave, 0, stream>>>(logits, AnyVec{correction, correction_dtype}, chosen, weight, total, top,
                                                   group_count, group_keep);
     LEONE_LAUNCH_CHECK("route_topk");
@@ -647,8 +666,8 @@ extern "C" int leone_route_plan(const float* logits, const void* correction, int
                   rows, total);
     LEONE_REQUIRE(top > 0 && top <= total, "route_plan: %d of %d outputs", top, total);
     LEONE_REQUIRE(!correction || correction_dtype == kF32 || correction_dtype == kBF16, "route_plan: unknown type of the correction");
-    LEONE_REQUIRE(group_count >= 1 && group_count <= kWave && total % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
-                  "route_plan: %d groups (at most %d, dividing %d outputs), %d kept", group_count, kWave, total, group_keep);
+    LEONE_REQUIRE(group_count >= 1 && total % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
+                  "route_plan: %d groups (dividing %d outputs), %d kept", group_count, total, group_keep);
     LEONE_REQUIRE(experts > 0 && experts <= 1024, "route_plan: %d experts (at most 1024)", experts);
     LEONE_REQUIRE(tile == kTilePairs || tile == 16 || tile == 64 || tile == 128, "route_plan: tiles of %d pairs", tile);
     const long pairs = static_cast<long>(rows) * top;

@@ -60,7 +60,7 @@ def make_engine(folder, dtype_name, **options):
     return Engine(load_model(folder, dtype_name), **options)
 
 
-def run_steps(engine, steps, spoil=False):
+def run_steps(engine, steps):
     from leone_amd.engine.engine import StepEntry
     outputs = {}
     for s in steps:
@@ -197,6 +197,52 @@ def test_trace_replay_as_a_user_runs_it(cases, tmp_path):
     compare(steps, outputs, expected, "float32", "trace replay")
 
 
+def test_command_line_generates_from_token_ids(tmp_path):
+    """``leone generate`` on a Zukinex folder: greedy tokens as the plain implementation picks them; ``leone
+    random-model`` writes a folder of the design that loads again."""
+    from leone_amd import cli
+    raw = zu.SMALL["B"]
+    weights = zu.make_weights(raw, 61, torch.float32, sharpen=2.0)
+    folder = zu.write_dir(str(tmp_path / "model"), raw, weights)
+    prompt = [5, 17, 3, 99, 42, 7]
+    out = str(tmp_path / "tokens.json")
+    assert cli.main(["generate", "-m", folder, "--prompt-tokens", ",".join(map(str, prompt)), "-n", "8", "--dtype", "float32",
+                     "--ignore-eos", "--debug-tokens", out]) == 0
+    with open(out) as handle:
+        got = json.load(handle)
+    tokens = list(prompt)
+    for token in got:
+        logits = plain.forward(raw, weights, tokens)[-1]
+        assert token == int(logits.argmax()) or float(logits.max() - logits[token]) < 1e-4
+        tokens.append(token)
+    assert len(got) == 8
+    config_path = str(tmp_path / "config.json")
+    with open(config_path, "w") as handle:
+        json.dump(zu.SMALL["A"], handle)
+    made = str(tmp_path / "made")
+    assert cli.main(["random-model", "--config", config_path, "--seed", "3", "--out", made]) == 0
+    engine = make_engine(made, "bfloat16", max_tokens=64)
+    from leone_amd.engine.engine import StepEntry
+    logits = engine.step([StepEntry("a", [1, 2, 3], [2])]).logits
+    assert logits.shape == (1, zu.SMALL["A"]["vocab"]) and torch.isfinite(logits).all()
+
+
+def test_which_attention_kernels_a_layer_gets(cases):
+    """Keys and values of one size that the matrix-core kernels take go to them in bfloat16, kept first keys and the
+    gate for every element included; values of another size, and float32, go to the row kernel."""
+    folder, _, _ = cases("C", "bfloat16")
+    engine = make_engine(folder, "bfloat16", max_tokens=256)
+    owner, reader = engine.model.layers[0].mixer, engine.model.layers[1].mixer
+    assert owner.keep_first == 4 and reader.keep_first == 2 and reader.shared_kv and owner.gate_each
+    assert owner.attention_kernels(torch.bfloat16, 16, 16) == {"decode": "split_kv", "prompt": "flash"}
+    assert reader.attention_kernels(torch.bfloat16, 16, 16) == {"decode": "split_kv", "prompt": "flash"}
+    assert owner.attention_kernels(torch.float32, 16, 16) == {"decode": "rows", "prompt": "rows"}
+    folder, _, _ = cases("A", "bfloat16")
+    other = make_engine(folder, "bfloat16", max_tokens=256).model.layers[0].mixer
+    assert other.value_dim != other.head_dim
+    assert other.attention_kernels(torch.bfloat16, 16, 16) == {"decode": "rows", "prompt": "rows"}
+
+
 # ---- each mechanism alone ---------------------------------------------------------------------------------------
 
 def close(have, want, tol, what):
@@ -274,6 +320,8 @@ ROUTERS = [{"experts": 6, "identity": 2, "top": 3, "groups": {"count": 4, "keep"
            {"experts": 9, "identity": 1, "top": 4, "groups": {"count": 5, "keep": 3}},
            {"experts": 60, "identity": 12, "top": 6, "groups": {"count": 8, "keep": 3}},
            {"experts": 140, "identity": 10, "top": 8, "groups": {"count": 10, "keep": 4}},
+           {"experts": 70, "identity": 3, "top": 2, "groups": {"count": 73, "keep": 22}},
+           {"experts": 200, "identity": 0, "top": 5, "groups": {"count": 100, "keep": 30}},
            {"experts": 4, "identity": 0, "top": 4, "groups": {"count": 1, "keep": 1}}]
 
 
