@@ -478,20 +478,27 @@ template <bool kGated>
 __global__ void __launch_bounds__(kMoeThreads, 2)
 moe_product_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y,
                          const float* __restrict__ pair_weight, const int* __restrict__ tile_expert,
-                         const int* __restrict__ tile_pairs, int top, int n, int k, int act) {
+                         const int* __restrict__ tile_pairs, int top, int n, int k, int act, int n_tiles, int n_blocks) {
     constexpr int kWRows = kGated ? 2 * kBigRows : kBigRows;          // rows of the matrix in a chunk
     constexpr int kXPieces = kBigPairs * 8 / kMoeThreads;             // 16-byte pieces of x a thread brings per chunk
     constexpr int kWPieces = kWRows * 8 / kMoeThreads;
     __shared__ uint4 sx[2 * kBigPairs * 4];                           // [half][row][4 pieces]
     __shared__ uint4 sw[2 * kWRows * 4];
-    const int tile = blockIdx.x;
+    // Workgroups go to the eight dies in turn, and each die has a cache of its own: the work is numbered so that a
+    // die gets a run of neighbouring (row block, tile) places, tiles fastest: the tiles of one expert, which read the
+    // same rows of its matrix, then lie on one die.
+    const int per_die = (n_tiles * n_blocks + 7) / 8;
+    const int place = static_cast<int>(blockIdx.x % 8) * per_die + static_cast<int>(blockIdx.x / 8);
+    if (place >= n_tiles * n_blocks) return;
+    const int tile = place % n_tiles;
+    const int row_block = place / n_tiles;
     const int e = tile_expert[tile];
     if (e < 0) return;
     const int tid = threadIdx.x;
     const int wave = tid / kWave, lane = tid % kWave;
     const int c = lane & 15, g = lane >> 4;
     const int wr = wave >> 1, wp = wave & 1;
-    const int row_base = blockIdx.y * kBigRows;
+    const int row_base = row_block * kBigRows;
     const long matrix = static_cast<long>(n) * k;
     const int* my_pairs = tile_pairs + static_cast<long>(tile) * kBigPairs;
 
@@ -718,12 +725,18 @@ extern "C" int leone_moe_product(const void* x, const void* w, void* y, const fl
         } else if (tile == 64) {
             if (gated) LEONE_MOE_CORES(4, 1, true);
             else LEONE_MOE_CORES(4, 1, false);
-        } else if (gated) {
-            moe_product_tiled_kernel<true><<<cores, kMoeThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y,
-                                                                              pair_weight, tile_expert, tile_pairs, top, n, k, act);
         } else {
-            moe_product_tiled_kernel<false><<<cores, kMoeThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y,
-                                                                               pair_weight, tile_expert, tile_pairs, top, n, k, act);
+            const long places = static_cast<long>(cores.x) * cores.y;
+            LEONE_REQUIRE(places + 7 <= 0x7fffffffL, "moe_product: too many tiles");
+            const int grid = static_cast<int>((places + 7) / 8 * 8);
+            if (gated)
+                moe_product_tiled_kernel<true><<<grid, kMoeThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w),
+                                                                                 y, pair_weight, tile_expert, tile_pairs, top, n, k, act,
+                                                                                 static_cast<int>(cores.x), static_cast<int>(cores.y));
+            else
+                moe_product_tiled_kernel<false><<<grid, kMoeThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w),
+                                                                                  y, pair_weight, tile_expert, tile_pairs, top, n, k, act,
+                                                                                  static_cast<int>(cores.x), static_cast<int>(cores.y));
         }
 #undef LEONE_MOE_CORES
         LEONE_LAUNCH_CHECK("moe_product");
