@@ -290,10 +290,11 @@ int leone_route_topk(const float* logits, const void* correction, int correction
 // 16, 64 or 128): tile_expert int32 [max_tiles] (-1: unused), tile_pairs int32 [max_tiles, tile] (-1: empty);
 // max_tiles >= min(pairs, pairs / tile + experts).
 int leone_moe_tile_pairs();
-// leone_route_topk and leone_moe_plan in one launch of one workgroup, for steps of at most 256 rows.
+// leone_route_topk and leone_moe_plan in one launch of one workgroup, for steps of at most 256 rows.  always: the last
+// so many of the experts are taken by every row with weight 1 (chosen and weight are [rows, top + always] then).
 int leone_route_plan(const float* logits, const void* correction, int correction_dtype, int* chosen, float* weight, int rows,
                      int total, int top, int group_count, int group_keep, int experts, int* tile_expert, int* tile_pairs,
-                     int max_tiles, int tile, hipStream_t stream);
+                     int max_tiles, int tile, int always, hipStream_t stream);
 int leone_moe_plan(const int* chosen, int pairs, int experts, int* tile_expert, int* tile_pairs, int max_tiles, int tile,
                    hipStream_t stream);
 // tile: leone_moe_tile_pairs() (any type and size), or 16, 64 or 128 (matrix cores: bfloat16, n and k multiples of 8).

@@ -44,7 +44,11 @@ __device__ inline void wave_best(float& v, int& at) {
 template <int kSlots>
 __device__ inline void route_row(int row, int lane, const float* __restrict__ logits, const AnyVec& correction,
                                  int* __restrict__ chosen, float* __restrict__ weight, int total, int top, int group_count,
-                                 int group_keep) {
+                                 int group_keep, int shift_from = 0x7fffffff, int always = 0) {
+    // `always` experts that every row takes with weight 1 stand behind the routed ones in the matrices (indices
+    // shift_from .. shift_from + always - 1): a row's places are its `top` choices and then these; a chosen router
+    // output from shift_from on (one that hands the row on) is numbered behind them.
+    const int places = top + always;
     const float* z = logits + static_cast<long>(row) * total;
     float s[kSlots], choice[kSlots];
     bool taken[kSlots];
@@ -154,17 +158,21 @@ __device__ inline void route_row(int row, int lane, const float* __restrict__ lo
             my_e = at;
         }
         if (n >= kWave && lane == 0) {       // more than 64 places: written as they come, scaled below
-            chosen[static_cast<long>(row) * top + n] = at;
-            weight[static_cast<long>(row) * top + n] = got;
+            chosen[static_cast<long>(row) * places + n] = at >= shift_from ? at + always : at;
+            weight[static_cast<long>(row) * places + n] = got;
         }
     }
     const float denom = picked_sum + 1e-20f;
     if (lane < top && lane < kWave) {
-        chosen[static_cast<long>(row) * top + lane] = my_e;
-        weight[static_cast<long>(row) * top + lane] = my_s / denom;
+        chosen[static_cast<long>(row) * places + lane] = my_e >= shift_from ? my_e + always : my_e;
+        weight[static_cast<long>(row) * places + lane] = my_s / denom;
     }
     if (top > kWave && lane == 0)
-        for (int n = kWave; n < top; ++n) weight[static_cast<long>(row) * top + n] /= denom;
+        for (int n = kWave; n < top; ++n) weight[static_cast<long>(row) * places + n] /= denom;
+    for (int i = lane; i < always; i += kWave) {
+        chosen[static_cast<long>(row) * places + top + i] = shift_from + i;
+        weight[static_cast<long>(row) * places + top + i] = 1.0f;
+    }
 }
 
 __global__ void __launch_bounds__(kWave)
@@ -221,17 +229,18 @@ moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int* __r
 __global__ void __launch_bounds__(1024)
 route_plan_kernel(const float* __restrict__ logits, AnyVec correction, int* __restrict__ chosen, float* __restrict__ weight,
                   int rows, int total, int top, int group_count, int group_keep, int experts, int* __restrict__ tile_expert,
-                  int* __restrict__ tile_pairs, int max_tiles, int tile) {
+                  int* __restrict__ tile_pairs, int max_tiles, int tile, int always) {
+    const int routed = experts - always;               // experts the router chooses among; the others every row takes
     __shared__ int count[1024];
     __shared__ int first_tile[1024];
     for (int row = threadIdx.x / kWave; row < rows; row += 1024 / kWave) {
         const int lane = threadIdx.x % kWave;
-        if (total <= kWave) route_row<1>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep);
-        else if (total <= 2 * kWave) route_row<2>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep);
-        else route_row<kRouteSlots>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep);
+        if (total <= kWave) route_row<1>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep, routed, always);
+        else if (total <= 2 * kWave) route_row<2>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep, routed, always);
+        else route_row<kRouteSlots>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep, routed, always);
     }
     __syncthreads();                                   // the choices are written; the same workgroup reads them
-    plan_tiles(chosen, rows * top, experts, tile_expert, tile_pairs, max_tiles, tile, count, first_tile);
+    plan_tiles(chosen, rows * (top + always), experts, tile_expert, tile_pairs, max_tiles, tile, count, first_tile);
 }
 
 template <typename T>
@@ -664,10 +673,14 @@ extern "C" int leone_route_topk(const float* logits, const void* correction, int
     return 0;
 }
 
-// leone_route_topk and leone_moe_plan in one launch (one workgroup: for steps of few rows).
+// leone_route_topk and leone_moe_plan in one launch (one workgroup: for steps of few rows).  `always`: the last so many
+// of the `experts` are taken by every row with weight 1 (a shared expert cut to the experts' size): chosen and weight are
+// [rows, top + always], a row's choices and then these; a chosen router output that stands for no matrix (from
+// experts - always on in the router's numbering) is numbered from `experts` on.
 extern "C" int leone_route_plan(const float* logits, const void* correction, int correction_dtype, int* chosen, float* weight,
                                 int rows, int total, int top, int group_count, int group_keep, int experts, int* tile_expert,
-                                int* tile_pairs, int max_tiles, int tile, hipStream_t stream) {
+                                int* tile_pairs, int max_tiles, int tile, int always, hipStream_t stream) {
+    LEONE_REQUIRE(always >= 0 && always < experts, "route_plan: %d of %d experts for every row", always, experts);
     LEONE_REQUIRE(logits && chosen && weight && tile_expert && tile_pairs, "route_plan: null pointer");
     LEONE_REQUIRE(rows > 0 && rows <= 256 && total > 0 && total <= kRouteSlots * kWave, "route_plan: rows %d (at most 256), %d router outputs",
                   rows, total);
@@ -677,12 +690,12 @@ extern "C" int leone_route_plan(const float* logits, const void* correction, int
                   "route_plan: %d groups (dividing %d outputs), %d kept", group_count, total, group_keep);
     LEONE_REQUIRE(experts > 0 && experts <= 1024, "route_plan: %d experts (at most 1024)", experts);
     LEONE_REQUIRE(tile == kTilePairs || tile == 16 || tile == 64 || tile == 128, "route_plan: tiles of %d pairs", tile);
-    const long pairs = static_cast<long>(rows) * top;
+    const long pairs = static_cast<long>(rows) * (top + always);
     const long needed = pairs / tile + experts;
     LEONE_REQUIRE(max_tiles >= (needed < pairs ? needed : pairs), "route_plan: %d tiles cannot hold %ld pairs of %d experts", max_tiles,
                   pairs, experts);
     route_plan_kernel<<<1, 1024, 0, stream>>>(logits, AnyVec{correction, correction_dtype}, chosen, weight, rows, total, top,
-                                              group_count, group_keep, experts, tile_expert, tile_pairs, max_tiles, tile);
+                                              group_count, group_keep, experts, tile_expert, tile_pairs, max_tiles, tile, always);
     LEONE_LAUNCH_CHECK("route_plan");
     return 0;
 }

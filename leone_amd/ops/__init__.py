@@ -1544,21 +1544,28 @@ def routed_experts(x: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, 
 
 def routed_feed_forward(x: torch.Tensor, logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, group_count: int,
                         group_keep: int, w_gate_up: torch.Tensor, w_down: torch.Tensor, activation: str = "silu",
-                        extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+                        extra: Optional[torch.Tensor] = None, always: int = 0) -> torch.Tensor:
     """``route_topk`` on the router's float32 ``logits`` and ``routed_experts`` with its choice; for steps of few rows
-    the choice and the tiles are made in one launch."""
+    (up to ``ROUTE_PLAN_ROWS``) the choice and the tiles are made in one launch.  ``always`` (such steps only): the
+    last so many experts of the matrices are no choice of the router's but taken by every row with weight 1 (a
+    shared expert cut to the experts' size rides along in the experts' launches)."""
     rows, hidden, experts, ff = _check_experts(x, w_gate_up, w_down)
     total = logits.shape[1]
     if rows > ROUTE_PLAN_ROWS:
+        if always:
+            raise KernelError(f"routed_feed_forward: experts for every row ride along in steps of up to {ROUTE_PLAN_ROWS} rows only")
         chosen, weight = route_topk(logits, correction, top, group_count, group_keep)
         return routed_experts(x, chosen, weight, w_gate_up, w_down, activation, extra)
     if total > library().leone_route_max_outputs():
         raise KernelError(f"route_topk: {total} router outputs, the kernel takes {library().leone_route_max_outputs()}")
-    tiles = _expert_tiles(x, rows, top, experts, hidden, ff)
-    chosen = torch.empty((rows, top), dtype=torch.int32, device=x.device)
-    weight = torch.empty((rows, top), dtype=torch.float32, device=x.device)
+    if not 0 <= always < experts:
+        raise KernelError(f"routed_feed_forward: {always} of {experts} experts for every row")
+    places = top + always
+    tiles = _expert_tiles(x, rows, places, experts, hidden, ff)
+    chosen = torch.empty((rows, places), dtype=torch.int32, device=x.device)
+    weight = torch.empty((rows, places), dtype=torch.float32, device=x.device)
     call("leone_route_plan", _dev(logits, "router logits", torch.float32, (rows, total)),
          _dev(correction, "router correction", None, (total,)), _code(correction, "router correction") if correction is not None else F32,
          _dev(chosen, "chosen"), _dev(weight, "weights"), rows, total, int(top), int(group_count), int(group_keep), experts,
-         _dev(tiles[2], "tiles"), _dev(tiles[3], "tile pairs"), tiles[1], tiles[0], _stream())
+         _dev(tiles[2], "tiles"), _dev(tiles[3], "tile pairs"), tiles[1], tiles[0], int(always), _stream())
     return _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, extra)

@@ -78,7 +78,7 @@ _PROTOTYPES = {
     "leone_attention_prefill_kept": [P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P, P,
                                      c_int, c_int, P],
     "leone_route_topk": [P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, P],
-    "leone_route_plan": [P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, c_int, c_int, P],
+    "leone_route_plan": [P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, c_int, c_int, c_int, P],
     "leone_moe_plan": [P, c_int, c_int, P, P, c_int, c_int, P],
     "leone_moe_product": [P, P, P, P, c_int, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "leone_moe_combine": [P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, P],

@@ -130,7 +130,8 @@ class RoutedGluMlp(Part):
             raise ValueError(f"unknown gate activation {self.activation!r}; known: {', '.join(ops.GATE_ACTIVATIONS)}")
         self.router_name, self.correction_name, self.expert_name = p["router"], p.get("correction"), p["expert"]
         self.shared = FEED_FORWARDS.build(p["shared"], **context) if p.get("shared") is not None else None
-        self.w_router = self.correction = self.w_gate_up = self.w_down = None
+        self.w_router = self.correction = self.w_gate_up = self.w_down = self.w_gate_up_all = self.w_down_all = None
+        self.always = 0
 
     def tensor_specs(self) -> List[TensorSpec]:
         specs = [TensorSpec(self.router_name, (self.total, self.hidden), MATRIX)]
@@ -148,8 +149,23 @@ class RoutedGluMlp(Part):
         self.correction = tensors.pop(self.correction_name).contiguous() if self.correction_name else None
         names = [self.expert_name.format(e=e) for e in range(self.experts)]
         # all experts side by side: [experts, 2, ff, hidden] (gate rows, then up rows) and [experts, hidden, ff]
-        self.w_gate_up = torch.stack([torch.stack([tensors.pop(n + ".gate"), tensors.pop(n + ".up")]) for n in names]).contiguous()
-        self.w_down = torch.stack([tensors.pop(n + ".down") for n in names]).contiguous()
+        gate_up = torch.stack([torch.stack([tensors.pop(n + ".gate"), tensors.pop(n + ".up")]) for n in names])
+        down = torch.stack([tensors.pop(n + ".down") for n in names])
+        # A shared expert of the experts' kind rides along in the experts' launches of short steps: cut into pieces of
+        # the experts' size (the last filled up with zero rows, which add nothing), they stand behind the experts as
+        # experts that every row takes with weight 1.
+        self.always = 0
+        if isinstance(self.shared, SwiGluMlp) and self.shared.activation == self.activation:
+            shared = {k: tensors[self.shared.names[k]] for k in ("gate", "up", "down")}
+            pieces = -(-self.shared.intermediate // self.intermediate)
+            pad = pieces * self.intermediate - self.shared.intermediate
+            rows = [torch.nn.functional.pad(shared[k], (0, 0, 0, pad)).view(pieces, self.intermediate, self.hidden) for k in ("gate", "up")]
+            cols = torch.nn.functional.pad(shared["down"], (0, pad)).view(self.hidden, pieces, self.intermediate).permute(1, 0, 2)
+            gate_up = torch.cat([gate_up, torch.stack(rows, dim=1).to(gate_up.dtype)])
+            down = torch.cat([down, cols.to(down.dtype)])
+            self.always = pieces
+        self.w_gate_up_all, self.w_down_all = gate_up.contiguous(), down.contiguous()
+        self.w_gate_up, self.w_down = self.w_gate_up_all[:self.experts], self.w_down_all[:self.experts]
         if self.shared is not None:
             self.shared.bind(tensors)
 
@@ -159,6 +175,9 @@ class RoutedGluMlp(Part):
     def forward(self, y: torch.Tensor, step: StepContext) -> torch.Tensor:
         y = ops.materialize(y)
         logits = ops.linear(y, self.w_router, out_dtype=torch.float32)
+        if self.always and y.shape[0] <= ops.ROUTE_PLAN_ROWS:
+            return ops.routed_feed_forward(y, logits, self.correction, self.top, self.group_count, self.group_keep,
+                                           self.w_gate_up_all, self.w_down_all, self.activation, always=self.always)
         extra = None
         if self.shared is not None:
             extra = self.shared.forward(y, step)
