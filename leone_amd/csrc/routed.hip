@@ -4,9 +4,13 @@
 //                equal groups of neighbours, a group's score its best choice score, only the best `keep` groups
 //                stay open (the others count as minus infinity); the `top` best open choice scores win; the
 //                weights are the winners' s over their sum (+ 1e-20).
-//   moe_plan     the (row, place) pairs of every expert gathered into tiles of kTilePairs pairs of one expert.
-//   moe_up       act(W_gate h) * (W_up h) of every pair, by its expert's matrices.
-//   moe_down     W_down of that, times the pair's weight, float.
+//   moe_plan     the (row, place) pairs of every expert gathered into tiles of pairs of one expert.
+//   route_plan   both in one launch of one workgroup, for steps of few rows; experts that every row takes with
+//                weight 1 (a shared expert cut to the experts' size) may stand behind the routed ones.
+//   moe_product  gated: act(W_gate x) * (W_up x) of every pair, by its expert's matrices; else W_down of that, times
+//                the pair's weight, float.  Three kernels: any type and size (float sums of 8-element runs a lane);
+//                bfloat16 on the matrix cores from registers (tiles of 16 or 64 pairs); bfloat16 on the matrix cores
+//                through shared memory (tiles of 128 pairs x 128 rows).
 //   moe_combine  a row's pairs summed in the order of its places; a router output beyond the experts with
 //                matrices hands the row itself on (times its weight); a delta that comes along is added.
 //
