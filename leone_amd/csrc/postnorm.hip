@@ -20,7 +20,34 @@ constexpr int kPostThreads = 256;
 //   gain2 == nullptr:  y[r] = x[r] in TY                               (y == nullptr: nothing is written)
 //   gain2 != nullptr:  y[i] = (x[r] / sqrt(mean(x[r]^2) + eps2)) * gain2, r = rows ? rows[i] : i
 // With `rows` the stream itself is left as it was (only some rows are looked at).
-template <typename TY>
+// kVec: elements a thread takes at a time (4 where the row's length and the addresses allow whole 16-byte runs).
+template <int kVec>
+__device__ inline void load_run(const float* p, float out[kVec]) {
+    if constexpr (kVec == 4) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+    } else {
+        out[0] = p[0];
+    }
+}
+template <int kVec>
+__device__ inline void store_run(float* p, const float v[kVec]) {
+    if constexpr (kVec == 4) *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+    else p[0] = v[0];
+}
+template <int kVec>
+__device__ inline void store_run(bf16_t* p, const float v[kVec]) {
+    if constexpr (kVec == 4) {
+        uint2 packed;
+        packed.x = bf16_bits_from_float(v[0]) | (static_cast<uint32_t>(bf16_bits_from_float(v[1])) << 16);
+        packed.y = bf16_bits_from_float(v[2]) | (static_cast<uint32_t>(bf16_bits_from_float(v[3])) << 16);
+        *reinterpret_cast<uint2*>(p) = packed;
+    } else {
+        p[0] = from_float<bf16_t>(v[0]);
+    }
+}
+
+template <typename TY, int kVec>
 __global__ void __launch_bounds__(kPostThreads)
 add_normed_kernel(float* __restrict__ x, const float* __restrict__ delta, int planes, long plane, AnyVec gain, float eps,
                   TY* __restrict__ y, AnyVec gain2, float eps2, const int* __restrict__ rows, int hidden) {
@@ -33,32 +60,50 @@ add_normed_kernel(float* __restrict__ x, const float* __restrict__ delta, int pl
     if (delta != nullptr) {
         const float* dr = delta + in_row * hidden;
         float ss = 0.f;
-        for (int c = threadIdx.x; c < hidden; c += kPostThreads) {
-            float d = dr[c];
-            for (int p = 1; p < planes; ++p) d += dr[p * plane + c];      // planes of a product cut along K, in order
-            row[c] = d;
-            ss = fmaf(d, d, ss);
+        for (int c = kVec * threadIdx.x; c < hidden; c += kVec * kPostThreads) {
+            float d[kVec];
+            load_run<kVec>(dr + c, d);
+            for (int p = 1; p < planes; ++p) {                 // planes of a product cut along K, in order
+                float more[kVec];
+                load_run<kVec>(dr + p * plane + c, more);
+#pragma unroll
+                for (int i = 0; i < kVec; ++i) d[i] += more[i];
+            }
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                row[c + i] = d[i];
+                ss = fmaf(d[i], d[i], ss);
+            }
         }
         inv = 1.0f / sqrtf(block_sum<kPostThreads>(ss, scratch) / static_cast<float>(hidden) + eps);
     }
     float ss2 = 0.f;
-    for (int c = threadIdx.x; c < hidden; c += kPostThreads) {
-        float v = xr[c];
+    for (int c = kVec * threadIdx.x; c < hidden; c += kVec * kPostThreads) {
+        float v[kVec];
+        load_run<kVec>(xr + c, v);
         if (delta != nullptr) {
-            v += (row[c] * inv) * load_any(gain, c);
-            if (!rows) xr[c] = v;
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) v[i] += (row[c + i] * inv) * load_any(gain, c + i);
+            if (!rows) store_run<kVec>(xr + c, v);
         }
         if (gain2.ptr != nullptr) {
-            row[c] = v;
-            ss2 = fmaf(v, v, ss2);
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                row[c + i] = v[i];
+                ss2 = fmaf(v[i], v[i], ss2);
+            }
         } else if (y != nullptr) {
-            y[static_cast<long>(out_row) * hidden + c] = from_float<TY>(v);
+            store_run<kVec>(y + static_cast<long>(out_row) * hidden + c, v);
         }
     }
     if (gain2.ptr == nullptr) return;
     const float inv2 = 1.0f / sqrtf(block_sum<kPostThreads>(ss2, scratch) / static_cast<float>(hidden) + eps2);
-    for (int c = threadIdx.x; c < hidden; c += kPostThreads)
-        y[static_cast<long>(out_row) * hidden + c] = from_float<TY>((row[c] * inv2) * load_any(gain2, c));
+    for (int c = kVec * threadIdx.x; c < hidden; c += kVec * kPostThreads) {
+        float v[kVec];
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) v[i] = (row[c + i] * inv2) * load_any(gain2, c + i);
+        store_run<kVec>(y + static_cast<long>(out_row) * hidden + c, v);
+    }
 }
 
 }  // namespace leone
@@ -81,12 +126,21 @@ extern "C" int leone_add_normed(float* x, const float* delta, int delta_planes, 
     LEONE_REQUIRE(delta || y, "add_normed: nothing to do");
     const AnyVec g1{gain, gain_dtype}, g2{gain2, gain2_dtype};
     const size_t shared = static_cast<size_t>(hidden) * sizeof(float);
-    if (y_dtype == kBF16 && y)
-        add_normed_kernel<bf16_t><<<n_rows, kPostThreads, shared, stream>>>(x, delta, delta_planes, delta_plane, g1, eps,
-                                                                           static_cast<bf16_t*>(y), g2, eps2, rows, hidden);
-    else
-        add_normed_kernel<float><<<n_rows, kPostThreads, shared, stream>>>(x, delta, delta_planes, delta_plane, g1, eps,
-                                                                          static_cast<float*>(y), g2, eps2, rows, hidden);
+    // whole 16-byte runs where the row's length, the planes' distance and every address allow them
+    const bool runs = hidden % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                      (!delta || (reinterpret_cast<uintptr_t>(delta) % 16 == 0 && (delta_planes == 1 || delta_plane % 4 == 0))) &&
+                      (!y || reinterpret_cast<uintptr_t>(y) % 16 == 0);
+#define LEONE_ADD_NORMED(TY, V)                                                                                        \
+    add_normed_kernel<TY, V><<<n_rows, kPostThreads, shared, stream>>>(x, delta, delta_planes, delta_plane, g1, eps,  \
+                                                                       static_cast<TY*>(y), g2, eps2, rows, hidden)
+    if (y_dtype == kBF16 && y) {
+        if (runs) LEONE_ADD_NORMED(bf16_t, 4);
+        else LEONE_ADD_NORMED(bf16_t, 1);
+    } else {
+        if (runs) LEONE_ADD_NORMED(float, 4);
+        else LEONE_ADD_NORMED(float, 1);
+    }
+#undef LEONE_ADD_NORMED
     LEONE_LAUNCH_CHECK("add_normed");
     return 0;
 }

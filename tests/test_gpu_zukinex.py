@@ -252,7 +252,7 @@ def close(have, want, tol, what):
     assert worst <= tol, f"{what}: off by {worst:.3e} of the largest value, bound {tol}"
 
 
-@pytest.mark.parametrize("hidden", [40, 192, 1000])
+@pytest.mark.parametrize("hidden", [40, 90, 192, 1000])
 def test_norm_behind_a_sublayer(hidden):
     """The norm of a sublayer's result, the sum into the stream and what the next product reads, in one kernel; at the
     model's end with the final norm on picked rows."""
