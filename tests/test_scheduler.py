@@ -264,7 +264,9 @@ def _loaded(seed, window=None, ahead=False):
     rng = random.Random(500 + seed)
     page_tokens = rng.choice([4, 8])
     groups = [GroupSpec(rng.choice([12, 16, 24]), page_tokens)]
-    if window:
+    if isinstance(window, tuple):                      # (window, first positions that stay when it passes)
+        groups.append(GroupSpec(14, page_tokens, window[0], window[1]))
+    elif window:
         groups.append(GroupSpec(12, page_tokens, window))
     cache = CacheManager(groups, 8, 4096)
     s = Scheduler(SchedulerPolicy(max_live_requests=4, prefill_chunk_tokens=rng.choice([3, 16, 64]),
@@ -285,7 +287,7 @@ def _loaded(seed, window=None, ahead=False):
 
 
 @pytest.mark.parametrize("ahead", [False, True])
-@pytest.mark.parametrize("window", [None, 9])
+@pytest.mark.parametrize("window", [None, 9, (9, 6), (5, 11)])
 @pytest.mark.parametrize("seed", range(4))
 def test_the_log_alone_shows_a_sound_run(seed, window, ahead):
     """Page conservation, budgets, one step in flight and contiguous positions are re-derived from the

@@ -88,7 +88,7 @@ def test_a_reader_of_another_layers_keys_runs_on_its_slot_and_widens_what_it_kee
 
 
 def test_a_window_that_passes_leaves_the_kept_first_pages():
-    cache = CacheManager([GroupSpec(12, 4, window=6, keep_first=5), GroupSpec(12, 4, window=6)], max_requests=2, max_context=48)
+    cache = CacheManager([GroupSpec(12, 4, window=6, keep_first=5), GroupSpec(12, 4, window=6)], max_requests=3, max_context=48)
     cache.admit("a")
     for tokens in (3, 7, 9, 1, 1, 10):
         cache.reserve("a", tokens)
@@ -98,6 +98,19 @@ def test_a_window_that_passes_leaves_the_kept_first_pages():
     assert [page >= 0 for page in cache.table("a", 0)] == [True, True, False, False, False, False, True, True]
     assert [page >= 0 for page in cache.table("a", 1)] == [False] * 6 + [True, True]
     assert cache.free_pages(0) == 8 and cache.free_pages(1) == 10
+    # a request that takes over another's 24 positions shares the kept first pages and the window's, nothing between
+    cache.admit("c")
+    cache.reserve("c", 24)
+    cache.commit("c", 24)
+    assert cache.fork("c", "d", 24) == 24
+    mine, theirs = cache.table("c", 0), cache.table("d", 0)
+    assert mine[2] == mine[3] == -1 and theirs == [mine[0], mine[1], -1, -1, mine[4], mine[5]]
+    assert cache.holders(0, mine[0]) == 2 and cache.holders(0, mine[5]) == 2
+    cache.check()
+    cache.release("c")
+    cache.check()
+    cache.release("d")
+    assert cache.free_pages(0) == 8
     cache.release("a")
     assert cache.free_pages(0) == 12
     cache.check()
